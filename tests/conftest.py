@@ -1,0 +1,34 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+def load_golden(name):
+    """Returns {case: {array_name: ndarray}} from tests/golden/<name>.npz."""
+    out = {}
+    with np.load(os.path.join(GOLDEN, name + ".npz")) as z:
+        for key in z.files:
+            case, arr = key.split("/")
+            out.setdefault(case, {})[arr] = z[key]
+    return out
+
+
+def rel_err(y, ref):
+    """max|y-ref| / max(|ref|, 1e-2*rms(ref)) -- the floor keeps zero crossings of y from
+    blowing a pointwise relative metric up."""
+    y = np.asarray(y, np.float64)
+    ref = np.asarray(ref, np.float64)
+    floor = 1e-2 * np.sqrt(np.mean(ref * ref)) + 1e-300
+    return float(np.max(np.abs(y - ref) / np.maximum(np.abs(ref), floor)))
