@@ -1,0 +1,166 @@
+"""Benchmark of the WKV hot path on one MI355X.
+
+A step = the Bi-WKV forward of one VRWKV-B backbone pass: 12 back-to-back calls (one per
+layer) at B=64, T=196, C=768, each on its own pre-generated seeded k, v (12 distinct buffer
+sets, 1.4 GB in fp32, so nothing stays cache-resident from call to call).  Inputs are resident
+in HBM before the timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--io fp32|bf16] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+LAYERS = 12
+B, T, C = 64, 196, 768
+
+
+def baseline_wu(torch):
+    import math
+    c = torch.arange(C, dtype=torch.float64)
+    w = (-5.0 + 8.0 * (c / (C - 1))) / T
+    u = (math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T
+    return w.float(), u.float()
+
+
+def cpu_baseline(torch, n_calls):
+    """The reference recurrence as PyTorch CPU-eager fp32 loops (oracle/torch_eager.py), timed on
+    a bounded sample of the same workload: n_calls full-shape calls."""
+    from oracle import torch_eager
+    w, u = baseline_wu(torch)
+    g = torch.Generator().manual_seed(1234)
+    k = torch.randn(B, T, C, generator=g)
+    v = torch.randn(B, T, C, generator=g)
+    torch_eager.biwkv_eager(w, u, k[:4], v[:4])          # warm-up
+    t0 = time.perf_counter()
+    for _ in range(n_calls):
+        y = torch_eager.biwkv_eager(w, u, k, v)
+    dt = time.perf_counter() - t0
+    bytes_alg = 3 * B * T * C * 4 + 2 * C * 4
+    return {
+        "value": round(n_calls * bytes_alg / dt / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{n_calls} calls at the full shape B={B} T={T} C={C} fp32 "
+                  f"(PyTorch CPU eager two-pass recurrence, {dt:.1f} s)",
+    }, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--io", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-calls", type=int, default=4)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
+                         "traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every sequence is independent; see "
+              "DESIGN.md for how the path would shard); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import vision_rwkv_amd as ops
+    from vision_rwkv_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    io = torch.float32 if args.io == "fp32" else torch.bfloat16
+    esz = 4 if args.io == "fp32" else 2
+    w, u = (t.to(dev) for t in baseline_wu(torch))
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    ks, vs = [], []
+    for _ in range(LAYERS):
+        ks.append(torch.randn(B, T, C, generator=g).to(dev).to(io))
+        vs.append(torch.randn(B, T, C, generator=g).to(dev).to(io))
+    ys = [torch.empty_like(k) for k in ks]
+
+    # direct C-ABI calls on torch's current stream (what ops.bi_wkv_forward does, minus the
+    # per-call output allocation)
+    L = ops.lib()
+    dt_code = _lib.VRWKV_F32 if args.io == "fp32" else _lib.VRWKV_BF16
+    ws_bytes = L.vrwkv_biwkv_fwd_workspace_bytes(B, T, C, dt_code)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    calls = [(w.data_ptr(), u.data_ptr(), ks[i].data_ptr(), vs[i].data_ptr(), ys[i].data_ptr(),
+              B, T, C, dt_code, ws.data_ptr() if ws_bytes else None, ws_bytes, stream.cuda_stream)
+             for i in range(LAYERS)]
+    fwd = L.vrwkv_biwkv_fwd
+
+    def step():
+        for a in calls:
+            rc = fwd(*a)
+            if rc:
+                _lib.check(rc)
+
+    if args.calibrate_copy:
+        ys[0].float().copy_(ks[0].float()) if args.io != "fp32" else ys[0].copy_(ks[0])
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = e0.elapsed_time(e1)
+    ms_per_step = max(dev_ms, 0.0) / args.steps
+    n_launch = args.steps * LAYERS
+    us_per_launch = dev_ms * 1e3 / n_launch
+    bytes_alg = 3 * B * T * C * esz + 2 * C * 4          # k, v read once, y written once, w and u
+    gbs = bytes_alg / (us_per_launch * 1e-6) / 1e9
+
+    out = {
+        "metric": "Bi-WKV fwd GB/s (% HBM peak) @VRWKV-B",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"Bi-WKV forward, VRWKV-B shape B={B} T={T} C={C}, {args.io} I/O, "
+                               f"{LAYERS} back-to-back calls per step on distinct seeded k,v",
+                   "io_dtype": args.io, "calls_per_step": LAYERS, "seed": 1234},
+        "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "us_per_call": round(us_per_launch, 3),
+        "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "biwkv_fwd_kernel (one launch per call)",
+            "algorithmic_bytes_per_launch": bytes_alg,
+        },
+    }
+    if not args.no_cpu_baseline:
+        cb, y_cpu = cpu_baseline(torch, args.cpu_calls)
+        out["cpu_baseline"] = cb
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,57 @@
+/* libvrwkv_hip.so -- C ABI of the MI355X (gfx950) WKV operators for Vision-RWKV.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its kernels on the
+ * HIP stream it is given (NULL = the default stream), returns without waiting for them,
+ * and never allocates or frees device memory: the caller owns every buffer, including
+ * the workspace whose size the *_workspace_bytes functions report.  No exception crosses
+ * this boundary; a non-zero status comes with a message in vrwkv_last_error().
+ *
+ * Layouts are the reference's: k, v, y, r, w_raw, gy, g* are (B,T,C) with C fastest and
+ * fully contiguous; per-channel parameters are (C,) -- for wkv6, u is (H,N) = (C,) -- fp32.
+ */
+#ifndef VRWKV_HIP_H
+#define VRWKV_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  Replaces TORCH_CHECK / assert at
+ * classification/mmcls_custom/models/backbones/cuda_new/bi_wkv.cpp:6-8,
+ * .../cuda_new/bi_wkv_kernel.cu:382-384 and .../cuda_v6/wkv6_cuda.cu:350-351. */
+enum {
+    VRWKV_OK = 0,
+    VRWKV_INVALID_ARG = 1,        /* null pointer, non-positive size, misaligned pointer */
+    VRWKV_UNSUPPORTED_DTYPE = 2,
+    VRWKV_UNSUPPORTED_SHAPE = 3,  /* e.g. C != H*64 for wkv6 */
+    VRWKV_LAUNCH_FAILED = 4,      /* hipGetLastError() after a launch */
+    VRWKV_WORKSPACE_TOO_SMALL = 5
+};
+
+/* Element type of the (B,T,C) tensors. */
+enum { VRWKV_F32 = 0, VRWKV_BF16 = 1, VRWKV_F16 = 2 };
+
+int vrwkv_version(void);                 /* major*10000 + minor*100 + patch */
+const char* vrwkv_last_error(void);      /* thread-local, never NULL */
+
+/* ---- Bi-WKV forward -------------------------------------------------------------------
+ * Replaces bi_wkv_forward(w,u,k,v) -> y
+ *   (classification/mmcls_custom/models/backbones/cuda_new/bi_wkv.cpp:23-33,
+ *    launcher .../cuda_new/bi_wkv_kernel.cu:370-399) and the legacy
+ *   forward(B,T,C,w,u,k,v,y) (.../backbones/cuda/wkv_op.cpp:6-8).
+ * w, u: (C,) fp32 (already divided by T by the caller, vrwkv.py:183).
+ * k, v, y: (B,T,C) of io_dtype; state and arithmetic are fp32.  No T_MAX and no
+ * C >= 32 / B*C % 32 restriction; T*C must stay below 2^29 elements.
+ * workspace: needed only for long sequences (see vrwkv_biwkv_fwd_workspace_bytes, which
+ * returns 0 when none is); may be NULL when that size is 0. */
+size_t vrwkv_biwkv_fwd_workspace_bytes(int B, int T, int C, int io_dtype);
+int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v, void* y,
+                    int B, int T, int C, int io_dtype,
+                    void* workspace, size_t workspace_bytes, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VRWKV_HIP_H */

@@ -1,0 +1,70 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header
+declares, and rejects bad arguments with a status and a message before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import vision_rwkv_amd
+    if not os.path.exists(vision_rwkv_amd.LIB_PATH):
+        vision_rwkv_amd.build(force=False)
+    return vision_rwkv_amd.lib()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "vrwkv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vrwkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_symbols()
+    assert "vrwkv_biwkv_fwd" in names and "vrwkv_last_error" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/vrwkv_hip.h but not exported"
+
+
+def test_version_and_error_string(lib):
+    assert lib.vrwkv_version() >= 100
+    assert isinstance(lib.vrwkv_last_error(), bytes)
+
+
+def test_argument_validation_without_device(lib):
+    f = lib.vrwkv_biwkv_fwd
+    one = ctypes.c_void_p(16)
+    # null pointers
+    assert f(None, None, None, None, None, 1, 1, 1, 0, None, 0, None) == 1
+    assert b"null" in lib.vrwkv_last_error()
+    # non-positive sizes
+    assert f(one, one, one, one, one, 0, 4, 4, 0, None, 0, None) == 1
+    assert f(one, one, one, one, one, 1, -3, 4, 0, None, 0, None) == 1
+    # unknown dtype code
+    assert f(one, one, one, one, one, 1, 4, 4, 7, None, 0, None) == 2
+    assert b"dtype" in lib.vrwkv_last_error()
+    # misaligned tensor pointer
+    assert f(one, one, ctypes.c_void_p(18), one, one, 1, 4, 4, 0, None, 0, None) == 1
+    # a long sequence needs the workspace the query reports
+    need = lib.vrwkv_biwkv_fwd_workspace_bytes(2, 4150, 768, 1)
+    assert need > 0
+    assert f(one, one, one, one, one, 2, 4150, 768, 1, None, 0, None) == 5
+    assert b"workspace" in lib.vrwkv_last_error()
+    assert lib.vrwkv_biwkv_fwd_workspace_bytes(64, 196, 768, 0) == 0
+    # too large for 32-bit buffer offsets
+    assert f(one, one, one, one, one, 1, 1 << 20, 1 << 10, 0, None, 0, None) == 3
+
+
+def test_python_boundary_errors_without_device():
+    import torch
+    import vision_rwkv_amd as ops
+    k = torch.randn(2, 8, 64)
+    w = torch.zeros(64)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ops.bi_wkv_forward(w, w, k, k)
+    with pytest.raises(TypeError):
+        ops.RUN_CUDA(w, w, k)

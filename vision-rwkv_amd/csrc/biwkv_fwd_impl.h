@@ -1,0 +1,723 @@
+// Bi-WKV forward for gfx950: kernels and launch plan (included by one .hip file per I/O type).
+//
+// Computes, per batch b and channel c (w, u already divided by T by the caller),
+//   y[t] = ( sum_{i!=t} e^{k_i - w(|t-i|-1)} v_i + e^{u+k_t} v_t ) / ( same with v -> 1 )
+// i.e. the formula evaluated by the in-chunk recurrence of
+// classification/mmcls_custom/models/backbones/cuda_new/bi_wkv_kernel.cu:93-108.
+//
+// Work decomposition (nothing like the reference's 32 token-chunks x 32 channels block):
+//   lane      = VEC adjacent channels  -> every load/store instruction of a wave touches
+//               one contiguous 64*VEC-element row segment of k, v or y;
+//   wave      = L consecutive tokens of those channels, held in registers;
+//   workgroup = S waves = S*L consecutive tokens (a "super-chunk") of 64*VEC channels;
+//   tile      = (batch, super-chunk, channel tile); workgroups are persistent and walk the
+//               tiles with stride gridDim.x, loading tile n+1 into a second register set
+//               while tile n is being computed, so HBM traffic overlaps the arithmetic.
+// k and v are read from HBM once: a wave keeps its L tokens in VGPRs between the
+// aggregate phase and the emit phase.  Only when T exceeds what one workgroup can hold
+// does a first kernel publish per-super-chunk aggregates to a small workspace and the
+// main kernel read the tokens a second time.
+// All tensor accesses are raw buffer loads/stores on a per-batch-element descriptor, so
+// tokens past T and channels past C are dropped by the hardware range check instead of
+// by exec-mask branches.
+//
+// Arithmetic is in the log2 domain (kappa = k*log2e, omega = w*log2e, mu = u*log2e) so
+// that every exponential is one v_exp_f32.
+//
+// Two code paths, chosen per tile from (w, u, T) alone and therefore identically by
+// every wave that touches a channel tile:
+//   fast   |omega|*(T+1) + |mu| <= 40.  One reference exponent R = max_t kappa_t per
+//          sequence; E_t = 2^(kappa_t-R) <= 1 is computed once per token and reused by
+//          both directions and both phases; states are plain decayed sums
+//          a <- g*a + E_t v_t (g = 2^-omega), no per-token max.  Under the bound every
+//          state stays within 2^+-41 of the largest term, so nothing overflows, and a
+//          term that underflows is below 2^-80 of its denominator.
+//   robust anything else: every state is a (num, den, exponent) triple renormalised at
+//          every token, exactly the reference's recurrence, for both directions.
+#pragma once
+#include "vrwkv_common.h"
+
+namespace vrwkv {
+namespace biwkv_fwd_detail {
+
+constexpr float FAST_LIMIT = 40.0f;
+constexpr int NSLOT = 6;   // workspace floats per (b, super-chunk, channel): A, B, pA|R, Cg, D, pC
+constexpr unsigned OOB_OFFSET = 0x80000000u;   // byte offset no descriptor here reaches
+constexpr unsigned CPOL_NT = 2;                // gfx94x/gfx950 cache policy bit: non-temporal (data streamed once)
+
+// Waves per workgroup: at most 8, i.e. two per SIMD, which leaves every wave 256 VGPRs -- enough
+// for the longest chunk (28 tokens: k, v, two partial arrays and the prefetched k, v of the next
+// tile, about 7 floats per token) without spilling.
+constexpr int smax_for(int L, int VEC) {
+    return (7 * L * VEC + 40 <= 256) ? 8 : 4;
+}
+
+// state <- decay-by-one-token(state) (+) token, all exponents in log2 units.
+__device__ __forceinline__ void tri_push(float& a, float& b, float& p, float om, float kap, float v) {
+    const float pw = fmaxf(p - om, NEG_BIG);
+    const float q = fmaxf(pw, kap);
+    const float e1 = fast_exp2(pw - q);
+    const float e2 = fast_exp2(kap - q);
+    a = e1 * a + e2 * v;
+    b = e1 * b + e2;
+    p = q;
+}
+// state <- decay-by-n-tokens(state) (+) other triple
+__device__ __forceinline__ void tri_merge(float& a, float& b, float& p, float om_n,
+                                          float a2, float b2, float p2) {
+    const float pw = fmaxf(p - om_n, NEG_BIG);
+    const float q = fmaxf(pw, p2);
+    const float e1 = fast_exp2(pw - q);
+    const float e2 = fast_exp2(p2 - q);
+    a = e1 * a + e2 * a2;
+    b = e1 * b + e2 * b2;
+    p = q;
+}
+
+// ---- raw buffer access: VEC elements of IO at byte offset voff (+ scalar soff) ----------
+template <int BYTES> struct BufRaw;
+template <> struct BufRaw<2> {
+    using type = unsigned short;
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b16(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b16(d, r, v, s, CP); }
+};
+template <> struct BufRaw<4> {
+    using type = unsigned int;
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b32(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b32(d, r, v, s, CP); }
+};
+template <> struct BufRaw<8> {
+    typedef unsigned int type __attribute__((ext_vector_type(2)));
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b64(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b64(d, r, v, s, CP); }
+};
+template <> struct BufRaw<16> {
+    typedef unsigned int type __attribute__((ext_vector_type(4)));
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b128(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b128(d, r, v, s, CP); }
+};
+
+// Raw (still packed) registers of one token: converted to fp32 only when consumed, so a
+// prefetched 16-bit tile costs half the registers.
+template <typename IO, int VEC> struct Packed { typename BufRaw<sizeof(IO) * VEC>::type raw; };
+
+template <typename IO, int VEC>
+__device__ __forceinline__ void unpack(const Packed<IO, VEC>& p, float (&out)[VEC]) {
+    IO tmp[VEC];
+    __builtin_memcpy(tmp, &p.raw, sizeof(p.raw));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) out[e] = to_f32(tmp[e]);
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, unsigned voff, const float (&in)[VEC]) {
+    IO tmp[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) tmp[e] = from_f32<IO>(in[e]);
+    typename BufRaw<sizeof(IO) * VEC>::type raw;
+    __builtin_memcpy(&raw, tmp, sizeof(raw));
+    BufRaw<sizeof(IO) * VEC>::template st<CPOL_NT>(raw, r, voff, 0);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+struct TileGeom {
+    int n_ctile, nSC, n_tiles;      // tile id = (b * nSC + sc) * n_ctile + ctile
+};
+
+// MODE 0: whole sequence in one workgroup.  MODE 1: aggregate-only pass of the long-
+// sequence path (writes the workspace).  MODE 2: emit pass of the long-sequence path.
+template <typename IO, int VEC, int L, int MODE>
+struct BiwkvTile {
+    static constexpr int SMAX = smax_for(L, VEC);
+    static constexpr int CH = WAVE * VEC;
+    using P = Packed<IO, VEC>;
+    typedef float (*AggPtr)[NSLOT][CH];
+
+    const float* __restrict__ w_;
+    const float* __restrict__ u_;
+    const IO* __restrict__ k_;
+    const IO* __restrict__ v_;
+    IO* __restrict__ y_;
+    float* __restrict__ ws;
+    int T, C;
+    TileGeom g;
+    int lane, wave, S;
+    AggPtr s_agg0, s_agg1;      // two LDS exchange buffers, alternated tile by tile
+
+    struct Where {
+        int b, sc, ctile, c0, tw;
+        bool cok;
+        unsigned voff0;          // byte offset of this lane's first token inside the batch slab
+        size_t slab;             // element offset of the batch slab
+    };
+
+    __device__ __forceinline__ Where locate(int tile) const {
+        Where q;
+        q.ctile = tile % g.n_ctile;
+        const int r = tile / g.n_ctile;
+        q.sc = r % g.nSC;
+        q.b = r / g.nSC;
+        q.c0 = (q.ctile * WAVE + lane) * VEC;
+        q.cok = q.c0 < C;
+        q.tw = (q.sc * S + wave) * L;
+        q.voff0 = q.cok ? (unsigned)(((size_t)q.tw * C + q.c0) * sizeof(IO)) : OOB_OFFSET;
+        q.slab = (size_t)q.b * T * C;
+        return q;
+    }
+
+    // Per-lane parameters of a tile, fetched together with its tokens so that consuming them
+    // never has to wait for the previous tile's stores.
+    struct WU { float w[VEC], u[VEC]; };
+
+    __device__ __forceinline__ void issue_wu(int tile, WU& wu) const {
+        const Where q = locate(tile);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            wu.w[e] = q.cok ? w_[q.c0 + e] : 0.f;
+            wu.u[e] = q.cok ? u_[q.c0 + e] : 0.f;
+        }
+    }
+    static __device__ __forceinline__ typename BufRaw<sizeof(IO) * VEC>::type load_raw(__amdgpu_buffer_rsrc_t r, unsigned vo) {
+        return BufRaw<sizeof(IO) * VEC>::template ld<CPOL_NT>(r, vo, 0);
+    }
+    __device__ __forceinline__ void issue_loads(int tile, P (&K)[L], P (&V)[L], WU& wu) const {
+        issue_wu(tile, wu);
+        const Where q = locate(tile);
+        const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + q.slab, bytes);
+        const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + q.slab, bytes);
+        const unsigned row = (unsigned)(C * sizeof(IO));
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            const unsigned vo = q.voff0 + (unsigned)j * row;
+            K[j].raw = load_raw(rk, vo);
+            V[j].raw = load_raw(rv, vo);
+        }
+    }
+
+    // Computes one tile from the packed registers K, V; in the middle (once K, V have been
+    // consumed) issues the loads of `next` into Kn, Vn when next < n_tiles.
+    // True when any channel of the tile is outside the plain-sum regime (wave-uniform, and the
+    // same for every wave and every super-chunk of a channel tile).
+    __device__ __forceinline__ bool tile_is_robust(const WU& wu, float (&om)[VEC], float (&mu)[VEC]) const {
+        bool bad = false;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            om[e] = wu.w[e] * LOG2E;
+            mu[e] = wu.u[e] * LOG2E;
+            bad = bad || !(fabsf(om[e]) * (float)(T + 1) + fabsf(mu[e]) <= FAST_LIMIT);
+        }
+#ifdef VRWKV_PROBE_NO_ROBUST
+        return false;
+#else
+        return __builtin_amdgcn_ballot_w64(bad) != 0ull;
+#endif
+    }
+
+    // Fast path of one tile from the packed registers K, V; in the middle (once K, V have been
+    // consumed) issues the loads of `next` into Kn, Vn when next < n_tiles.  Tiles that need
+    // the robust path are skipped here and handled by run_robust() afterwards.
+    // Consecutive tiles alternate between the two LDS buffers (`par`), so one barrier per
+    // exchange is enough: a wave can only write buffer `par` again after passing a barrier of
+    // the tile in between, which every wave reaches after its last read of this tile.
+    __device__ __forceinline__ void run(int tile, int next, int par, P (&K)[L], P (&V)[L], const WU& wu,
+                                        P (&Kn)[L], P (&Vn)[L], WU& wun) const {
+        const Where q = locate(tile);
+        const AggPtr s_agg = par ? s_agg1 : s_agg0;
+        const float NEG_INF = -__builtin_inff();
+        const int nSC = g.nSC;
+        const int li = lane * VEC;
+
+        float om[VEC], mu[VEC];
+        if (tile_is_robust(wu, om, mu)) {
+            if (next < g.n_tiles) issue_loads(next, Kn, Vn, wun);
+            return;
+        }
+
+        const unsigned row = (unsigned)(C * sizeof(IO));
+        const __amdgpu_buffer_rsrc_t ry = make_rsrc(y_ + q.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+        const size_t ws_b = (size_t)q.b * nSC * NSLOT * C;
+        auto ws_at = [&](int s, int slot, int e) -> float& {
+            return ws[ws_b + ((size_t)s * NSLOT + slot) * C + q.c0 + e];
+        };
+        // The next tile is fetched a token at a time behind the arithmetic (k during the
+        // aggregate pass, v during the ascending sweep): few vector-memory instructions are
+        // outstanding per CU at any moment, so issuing them never stalls the wave for long.
+        const bool have_next = next < g.n_tiles;
+        const Where qn = locate(have_next ? next : tile);
+        const __amdgpu_buffer_rsrc_t rkn = make_rsrc(k_ + qn.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+        const __amdgpu_buffer_rsrc_t rvn = make_rsrc(v_ + qn.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+        if (have_next) issue_wu(next, wun);
+
+        // unpack; tokens past T read as zero from the buffer and get k = -inf here
+        float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            unpack<IO, VEC>(K[j], X0[j]);
+            unpack<IO, VEC>(V[j], X1[j]);
+            const bool tok = q.tw + j < T;               // wave-uniform
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) X0[j][e] = tok ? X0[j][e] : NEG_INF;
+        }
+
+        // ================================== fast path ==================================
+        // ONE workgroup barrier per tile:
+        //  1. the wave takes its own reference exponent Rw = ceil(max kappa over its L tokens),
+        //     forms E = 2^(kappa-Rw) <= 1 and E*v, and its two chunk aggregates in units of 2^Rw;
+        //  2. it publishes (A, B, Cg, D, Rw); barrier; every wave reads all S entries at once;
+        //  3. R = max Rw.  All Rw are integers, so bringing another wave's aggregate to the common
+        //     scale is an exact ldexp (no exponential); the carry-in is accumulated at scale 2^R
+        //     and then shifted to the wave's own scale 2^Rw, in which the sweeps run unchanged
+        //     (y is a ratio, the scale cancels).  The shift is capped at 2^100: beyond that the
+        //     wave's own terms are below 2^-60 of the carry and the cap only keeps fp32 finite.
+        float gd[VEC], Rw[VEC], Rpub[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            gd[e] = fast_exp2(-om[e]);
+            float m = NEG_INF;
+#pragma unroll
+            for (int j = 0; j < L; ++j) m = fmaxf(m, X0[j][e]);
+            const bool any = m > NEG_INF;
+            Rw[e] = any ? ceilf(m * LOG2E) : 0.f;
+            Rpub[e] = any ? Rw[e] : NEG_BIG;              // a wave with no token must not set the scale
+        }
+        float A[VEC], Bd[VEC], Cg[VEC], D[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { A[e] = 0.f; Bd[e] = 0.f; Cg[e] = 0.f; D[e] = 0.f; }
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                // one rounding for k*log2e - Rw: the heaviest tokens have the smallest argument
+                const float E = fast_exp2(fmaf(X0[j][e], LOG2E, -Rw[e]));
+                X0[j][e] = E;
+                X1[j][e] = E * X1[j][e];
+                A[e] = fmaf(gd[e], A[e], X1[j][e]);       // referenced to the chunk end
+                Bd[e] = fmaf(gd[e], Bd[e], E);
+            }
+            if (have_next) Kn[j].raw = load_raw(rkn, qn.voff0 + (unsigned)j * row);
+        }
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                Cg[e] = fmaf(gd[e], Cg[e], X1[j][e]);      // referenced to the chunk start
+                D[e] = fmaf(gd[e], D[e], X0[j][e]);
+            }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            s_agg[wave][0][li + e] = A[e];
+            s_agg[wave][1][li + e] = Bd[e];
+            s_agg[wave][2][li + e] = Rpub[e];
+            s_agg[wave][3][li + e] = Cg[e];
+            s_agg[wave][4][li + e] = D[e];
+        }
+        lds_barrier();
+
+        float G[VEC];                                     // decay over one wave's chunk
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) G[e] = fast_exp2(-om[e] * (float)L);
+        auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
+
+        float a[VEC], bb[VEC], c[VEC], d[VEC], R[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            // all reads are issued before the dependent steps (one LDS latency, not S of them)
+            float la[SMAX], lb[SMAX], lc[SMAX], ld[SMAX], lr[SMAX];
+#pragma unroll
+            for (int s = 0; s < SMAX; ++s) {
+                const int ss = s < S ? s : S - 1;
+                la[s] = s_agg[ss][0][li + e];
+                lb[s] = s_agg[ss][1][li + e];
+                lr[s] = s_agg[ss][2][li + e];
+                lc[s] = s_agg[ss][3][li + e];
+                ld[s] = s_agg[ss][4][li + e];
+            }
+            float r = NEG_BIG;
+#pragma unroll
+            for (int s = 0; s < SMAX; ++s) r = fmaxf(r, lr[s]);
+            if (MODE == 2) {
+                r = NEG_BIG;
+                if (q.cok) for (int s = 0; s < nSC; ++s) r = fmaxf(r, ws_at(s, 2, e));
+            }
+            r = (r > NEG_BIG) ? r : 0.f;
+            R[e] = r;
+            float aa = 0.f, ab = 0.f, ac = 0.f, ad = 0.f;
+            if (MODE == 1) {
+                // fold all S wave aggregates into the super-chunk aggregate (published by wave 0)
+#pragma unroll
+                for (int s = 0; s < SMAX; ++s)
+                    if (s < S) {
+                        const int sh = shift_of(lr[s], r);
+                        aa = fmaf(G[e], aa, ldexpf(la[s], sh));
+                        ab = fmaf(G[e], ab, ldexpf(lb[s], sh));
+                    }
+#pragma unroll
+                for (int s = SMAX - 1; s >= 0; --s)
+                    if (s < S) {
+                        const int sh = shift_of(lr[s], r);
+                        ac = fmaf(G[e], ac, ldexpf(lc[s], sh));
+                        ad = fmaf(G[e], ad, ldexpf(ld[s], sh));
+                    }
+            } else {
+                if (MODE == 2 && q.cok) {
+                    const float GS = fast_exp2(-om[e] * (float)(S * L));
+                    for (int s = 0; s < q.sc; ++s) {
+                        const int sh = shift_of(ws_at(s, 2, e), r);
+                        aa = fmaf(GS, aa, ldexpf(ws_at(s, 0, e), sh));
+                        ab = fmaf(GS, ab, ldexpf(ws_at(s, 1, e), sh));
+                    }
+                    for (int s = nSC - 1; s > q.sc; --s) {
+                        const int sh = shift_of(ws_at(s, 2, e), r);
+                        ac = fmaf(GS, ac, ldexpf(ws_at(s, 3, e), sh));
+                        ad = fmaf(GS, ad, ldexpf(ws_at(s, 4, e), sh));
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < SMAX; ++s)
+                    if (s < wave) {                      // wave-uniform
+                        const int sh = shift_of(lr[s], r);
+                        aa = fmaf(G[e], aa, ldexpf(la[s], sh));
+                        ab = fmaf(G[e], ab, ldexpf(lb[s], sh));
+                    }
+#pragma unroll
+                for (int s = SMAX - 1; s >= 0; --s)
+                    if (s > wave && s < S) {
+                        const int sh = shift_of(lr[s], r);
+                        ac = fmaf(G[e], ac, ldexpf(lc[s], sh));
+                        ad = fmaf(G[e], ad, ldexpf(ld[s], sh));
+                    }
+                // to the wave's own scale
+                const int up = (int)fminf(r - Rw[e], 100.f);
+                aa = ldexpf(aa, up); ab = ldexpf(ab, up); ac = ldexpf(ac, up); ad = ldexpf(ad, up);
+            }
+            a[e] = aa; bb[e] = ab; c[e] = ac; d[e] = ad;
+        }
+
+        if (MODE == 1) {
+            if (wave == 0 && q.cok) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    ws_at(q.sc, 0, e) = a[e];
+                    ws_at(q.sc, 1, e) = bb[e];
+                    ws_at(q.sc, 2, e) = R[e];
+                    ws_at(q.sc, 3, e) = c[e];
+                    ws_at(q.sc, 4, e) = d[e];
+                    ws_at(q.sc, 5, e) = R[e];
+                }
+            }
+            if (have_next) {
+#pragma unroll
+                for (int j = 0; j < L; ++j) Vn[j].raw = load_raw(rvn, qn.voff0 + (unsigned)j * row);
+            }
+            return;
+        }
+
+        // emit: ascending sweep leaves past + bonus partials, descending sweep adds the future
+        float cu[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) cu[e] = fast_exp2(mu[e]);
+        float PN[L][VEC], PD[L][VEC];
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                PN[j][e] = fmaf(cu[e], X1[j][e], a[e]);
+                PD[j][e] = fmaf(cu[e], X0[j][e], bb[e]);
+                a[e] = fmaf(gd[e], a[e], X1[j][e]);
+                bb[e] = fmaf(gd[e], bb[e], X0[j][e]);
+            }
+            if (have_next) Vn[j].raw = load_raw(rvn, qn.voff0 + (unsigned)j * row);
+        }
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j) {
+            float out[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                out[e] = (PN[j][e] + c[e]) * fast_rcp(PD[j][e] + d[e]);
+                c[e] = fmaf(gd[e], c[e], X1[j][e]);
+                d[e] = fmaf(gd[e], d[e], X0[j][e]);
+            }
+            buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
+        }
+    }
+
+    // Robust path of one tile, self-contained (own loads, no prefetch); a no-op for tiles the
+    // fast path has already done.  Ends with a barrier so that the LDS buffer can be reused.
+    __device__ __forceinline__ void run_robust(int tile) const {
+        const Where q = locate(tile);
+        const AggPtr s_agg = s_agg0;
+        const float NEG_INF = -__builtin_inff();
+        const int nSC = g.nSC;
+        const int li = lane * VEC;
+        float om[VEC], mu[VEC];
+        WU wu;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            wu.w[e] = q.cok ? w_[q.c0 + e] : 0.f;
+            wu.u[e] = q.cok ? u_[q.c0 + e] : 0.f;
+        }
+        if (!tile_is_robust(wu, om, mu)) return;
+
+        const unsigned row = (unsigned)(C * sizeof(IO));
+        const __amdgpu_buffer_rsrc_t ry = make_rsrc(y_ + q.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+        const size_t ws_b = (size_t)q.b * nSC * NSLOT * C;
+        auto ws_at = [&](int s, int slot, int e) -> float& {
+            return ws[ws_b + ((size_t)s * NSLOT + slot) * C + q.c0 + e];
+        };
+        float X0[L][VEC], X1[L][VEC];
+        {
+            P K[L], V[L];
+            WU unused;
+            issue_loads(tile, K, V, unused);
+#pragma unroll
+            for (int j = 0; j < L; ++j) {
+                unpack<IO, VEC>(K[j], X0[j]);
+                unpack<IO, VEC>(V[j], X1[j]);
+                const bool tok = q.tw + j < T;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) X0[j][e] = tok ? X0[j][e] * LOG2E : NEG_INF;
+            }
+        }
+        // ================================== robust path ==================================
+        float A[VEC], Bd[VEC], pA[VEC], Cg[VEC], D[VEC], pC[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            A[e] = 0.f; Bd[e] = 0.f; pA[e] = NEG_BIG; Cg[e] = 0.f; D[e] = 0.f; pC[e] = NEG_BIG;
+        }
+#pragma unroll
+        for (int j = 0; j < L; ++j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) tri_push(A[e], Bd[e], pA[e], om[e], X0[j][e], X1[j][e]);
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) tri_push(Cg[e], D[e], pC[e], om[e], X0[j][e], X1[j][e]);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            s_agg[wave][0][li + e] = A[e];
+            s_agg[wave][1][li + e] = Bd[e];
+            s_agg[wave][2][li + e] = pA[e];
+            s_agg[wave][3][li + e] = Cg[e];
+            s_agg[wave][4][li + e] = D[e];
+            s_agg[wave][5][li + e] = pC[e];
+        }
+        lds_barrier();
+
+        if (MODE == 1) {
+            if (wave == 0 && q.cok) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float omL = om[e] * (float)L;
+                    float a = 0.f, bb = 0.f, p = NEG_BIG, c = 0.f, d = 0.f, o = NEG_BIG;
+                    for (int s = 0; s < S; ++s)
+                        tri_merge(a, bb, p, omL, s_agg[s][0][li + e], s_agg[s][1][li + e], s_agg[s][2][li + e]);
+                    for (int s = S - 1; s >= 0; --s)
+                        tri_merge(c, d, o, omL, s_agg[s][3][li + e], s_agg[s][4][li + e], s_agg[s][5][li + e]);
+                    ws_at(q.sc, 0, e) = a; ws_at(q.sc, 1, e) = bb; ws_at(q.sc, 2, e) = p;
+                    ws_at(q.sc, 3, e) = c; ws_at(q.sc, 4, e) = d;  ws_at(q.sc, 5, e) = o;
+                }
+            }
+            lds_barrier();
+            return;
+        }
+
+        float a[VEC], bb[VEC], p[VEC], c[VEC], d[VEC], o[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            a[e] = 0.f; bb[e] = 0.f; p[e] = NEG_BIG; c[e] = 0.f; d[e] = 0.f; o[e] = NEG_BIG;
+        }
+        if (MODE == 2 && q.cok) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float omSL = om[e] * (float)(S * L);
+                for (int s = 0; s < q.sc; ++s)
+                    tri_merge(a[e], bb[e], p[e], omSL, ws_at(s, 0, e), ws_at(s, 1, e), ws_at(s, 2, e));
+                for (int s = nSC - 1; s > q.sc; --s)
+                    tri_merge(c[e], d[e], o[e], omSL, ws_at(s, 3, e), ws_at(s, 4, e), ws_at(s, 5, e));
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float omL = om[e] * (float)L;
+            for (int s = 0; s < wave; ++s)
+                tri_merge(a[e], bb[e], p[e], omL, s_agg[s][0][li + e], s_agg[s][1][li + e], s_agg[s][2][li + e]);
+            for (int s = S - 1; s > wave; --s)
+                tri_merge(c[e], d[e], o[e], omL, s_agg[s][3][li + e], s_agg[s][4][li + e], s_agg[s][5][li + e]);
+        }
+
+        float PN[L][VEC], PD[L][VEC], PM[L][VEC];
+#pragma unroll
+        for (int j = 0; j < L; ++j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float uk = mu[e] + X0[j][e];
+                const float pm = fmaxf(p[e], uk);
+                const float ea = fast_exp2(p[e] - pm);
+                const float eu = fast_exp2(uk - pm);
+                PN[j][e] = ea * a[e] + eu * X1[j][e];
+                PD[j][e] = ea * bb[e] + eu;
+                PM[j][e] = pm;
+                tri_push(a[e], bb[e], p[e], om[e], X0[j][e], X1[j][e]);
+            }
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j) {
+            float out[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float m = fmaxf(PM[j][e], o[e]);
+                const float e1 = fast_exp2(PM[j][e] - m);
+                const float e2 = fast_exp2(o[e] - m);
+                out[e] = (e1 * PN[j][e] + e2 * c[e]) / (e1 * PD[j][e] + e2 * d[e]);
+                tri_push(c[e], d[e], o[e], om[e], X0[j][e], X1[j][e]);
+            }
+            buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);
+        }
+        lds_barrier();
+    }
+};
+
+
+template <typename IO, int VEC, int L, int MODE>
+__global__ __launch_bounds__(smax_for(L, VEC) * WAVE)
+void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
+                      const IO* __restrict__ k_, const IO* __restrict__ v_, IO* __restrict__ y_,
+                      float* __restrict__ ws, int T, int C, TileGeom g)
+{
+    using Tile = BiwkvTile<IO, VEC, L, MODE>;
+    __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
+
+    Tile t;
+    t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
+    t.T = T; t.C = C; t.g = g;
+    t.lane = threadIdx.x & (WAVE - 1);
+    t.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    t.S = blockDim.x >> 6;
+    t.s_agg0 = s_agg[0];
+    t.s_agg1 = s_agg[1];
+
+    typename Tile::P K0[L], V0[L], K1[L], V1[L];
+    typename Tile::WU wu0, wu1;
+    int tile = blockIdx.x;
+    if (tile >= g.n_tiles) return;
+    t.issue_loads(tile, K0, V0, wu0);
+    for (;;) {
+        int next = tile + gridDim.x;
+        t.run(tile, next, 0, K0, V0, wu0, K1, V1, wu1);
+        if (next >= g.n_tiles) break;
+        tile = next;
+        next = tile + gridDim.x;
+        t.run(tile, next, 1, K1, V1, wu1, K0, V0, wu0);
+        if (next >= g.n_tiles) break;
+        tile = next;
+    }
+    // second walk: tiles whose parameters need the renormalising recurrence
+    lds_barrier();
+    for (tile = blockIdx.x; tile < g.n_tiles; tile += gridDim.x) t.run_robust(tile);
+}
+
+// ------------------------------- host-side dispatch ---------------------------------
+struct Plan {
+    int L = 0, S = 0, nSC = 0, VEC = 0, grid = 0;
+    TileGeom geom{};
+    bool multi() const { return nSC > 1; }
+};
+
+constexpr int kLs[] = {4, 8, 16, 28};
+constexpr int kNumL = sizeof(kLs) / sizeof(kLs[0]);
+
+inline int env_int(const char* name) {
+    const char* s = getenv(name);
+    return s ? atoi(s) : 0;
+}
+
+inline int num_cus() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+inline Plan make_plan(int B, int T, int C, int io_dtype) {
+    Plan p;
+    (void)io_dtype;
+    const int el = env_int("VRWKV_BIWKV_L");              // tuning overrides
+    const int es = env_int("VRWKV_BIWKV_S");
+    p.VEC = 1;
+    int best = -1, best_waste = 1 << 30;
+    for (int i = 0; i < kNumL; ++i) {
+        const int L = kLs[i];
+        if (el && L != el) continue;
+        const int S = (T + L - 1) / L;
+        if (S > smax_for(L, p.VEC)) continue;
+        const int waste = S * L - T;
+        if (waste < best_waste) { best = i; best_waste = waste; }
+    }
+    if (best >= 0) {
+        p.L = kLs[best];
+        p.S = (T + p.L - 1) / p.L;
+        p.nSC = 1;
+    } else {
+        p.L = 28;
+        for (int i = 0; i < kNumL; ++i) if (el == kLs[i]) p.L = el;
+        p.S = smax_for(p.L, p.VEC);
+        if (es >= 1 && es <= smax_for(p.L, p.VEC)) p.S = es;
+        p.nSC = (T + p.S * p.L - 1) / (p.S * p.L);
+    }
+    const int cap = smax_for(p.L, p.VEC);
+    p.geom.n_ctile = (C + WAVE * p.VEC - 1) / (WAVE * p.VEC);
+    p.geom.nSC = p.nSC;
+    p.geom.n_tiles = B * p.nSC * p.geom.n_ctile;
+    // persistent grid: as many workgroups as can be resident at once
+    const int wg_per_cu = (cap / p.S) > 0 ? (cap / p.S) : 1;
+    int grid = num_cus() * wg_per_cu;
+    const int eg = env_int("VRWKV_BIWKV_GRID");
+    if (eg > 0) grid = eg;
+    p.grid = grid < p.geom.n_tiles ? grid : p.geom.n_tiles;
+    return p;
+}
+
+template <typename IO, int VEC, int L>
+int launch_L(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+             float* ws, int B, int T, int C, hipStream_t st) {
+    const dim3 block(p.S * WAVE);
+    const dim3 grid(p.grid);
+    const IO* kk = static_cast<const IO*>(k);
+    const IO* vv = static_cast<const IO*>(v);
+    IO* yy = static_cast<IO*>(y);
+    if (!p.multi()) {
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+    } else {
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+    }
+    return check_launch("biwkv_fwd");
+}
+
+template <typename IO, int VEC>
+int launch_VEC(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+               float* ws, int B, int T, int C, hipStream_t st) {
+    switch (p.L) {
+#define VRWKV_CASE(LL) case LL: return launch_L<IO, VEC, LL>(p, w, u, k, v, y, ws, B, T, C, st); break;
+        VRWKV_CASE(4) VRWKV_CASE(8) VRWKV_CASE(16) VRWKV_CASE(28)
+#undef VRWKV_CASE
+    }
+    set_error("biwkv_fwd: internal error, no kernel for L=%d VEC=%d", p.L, VEC);
+    return VRWKV_INVALID_ARG;
+}
+
+template <typename IO>
+int biwkv_fwd_launch_io(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+                        float* ws, int B, int T, int C, hipStream_t st) {
+    return launch_VEC<IO, 1>(p, w, u, k, v, y, ws, B, T, C, st);
+}
+
+}  // namespace biwkv_fwd_detail
+}  // namespace vrwkv

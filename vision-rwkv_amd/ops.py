@@ -1,0 +1,101 @@
+"""Operator boundary: the reference's autograd Functions and RUN_* entry points, backed by
+libvrwkv_hip.so.
+
+Mirrors
+  WKV / RUN_CUDA(w,u,k,v)                 classification/mmcls_custom/models/backbones/vrwkv.py:29-65
+  legacy RUN_CUDA(B,T,C,w,u,k,v)          classification/mae/vrwkv/vrwkv.py:30-90
+with the same argument meaning, output dtype rule and error behaviour (RuntimeError for
+non-device / non-contiguous tensors).
+"""
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.VRWKV_F32, torch.bfloat16: _lib.VRWKV_BF16, torch.float16: _lib.VRWKV_F16}
+
+
+def _check_input(x, name):
+    # CHECK_INPUT of bi_wkv.cpp:6-8
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def bi_wkv_forward(w, u, k, v):
+    """Extension-level entry (bi_wkv.cpp:23-33): w,u (C,) fp32; k,v (B,T,C) of one dtype
+    (fp32, bf16 or fp16); returns y (B,T,C) of that dtype.  State and arithmetic are fp32."""
+    for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v")):
+        _check_input(t, n)
+    if k.dim() != 3 or v.shape != k.shape:
+        raise RuntimeError("k and v must both be (B,T,C)")
+    B, T, C = k.shape
+    if w.numel() != C or u.numel() != C:
+        raise RuntimeError("w and u must have C elements")
+    if w.dtype != torch.float32 or u.dtype != torch.float32:
+        raise RuntimeError("w and u must be float32")
+    if k.dtype not in _DT or v.dtype != k.dtype:
+        raise RuntimeError("k and v must share one of float32 / bfloat16 / float16")
+    L = _lib.lib()
+    dt = _DT[k.dtype]
+    y = torch.empty_like(k)
+    if y.numel() == 0:
+        return y
+    ws_bytes = L.vrwkv_biwkv_fwd_workspace_bytes(B, T, C, dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=k.device) if ws_bytes else None
+    with torch.cuda.device(k.device):
+        _lib.check(L.vrwkv_biwkv_fwd(w.data_ptr(), u.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
+                                     B, T, C, dt, ws.data_ptr() if ws is not None else None, ws_bytes,
+                                     _stream_ptr(k.device)))
+    return y
+
+
+class WKV(torch.autograd.Function):
+    """Bi-WKV with the reference's dtype rule: arithmetic in fp32, the result is fp32 unless
+    the *parameter* w is half / bfloat16, in which case it has w's dtype (vrwkv.py:31-44).
+    When k and v already arrive in that 16-bit dtype they are consumed as they are
+    (no up-cast copies, no separate down-cast of y)."""
+
+    @staticmethod
+    def forward(ctx, w, u, k, v):
+        ctx.save_for_backward(w, u, k, v)
+        out_dtype = w.dtype if w.dtype in (torch.half, torch.bfloat16) else torch.float32
+        wf = w.float().contiguous()
+        uf = u.float().contiguous()
+        if k.dtype == out_dtype and v.dtype == out_dtype:
+            return bi_wkv_forward(wf, uf, k.contiguous(), v.contiguous())
+        y = bi_wkv_forward(wf, uf, k.float().contiguous(), v.float().contiguous())
+        return y if out_dtype == torch.float32 else y.to(out_dtype)
+
+    @staticmethod
+    def backward(ctx, gy):
+        raise NotImplementedError("Bi-WKV backward is not built yet in this library")
+
+
+class _WKVLegacy(torch.autograd.Function):
+    """Seven-argument form used by the MAE code (classification/mae/vrwkv/vrwkv.py:30-90)."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, w, u, k, v):
+        if tuple(k.shape) != (B, T, C):
+            raise RuntimeError(f"k has shape {tuple(k.shape)}, expected {(B, T, C)}")
+        return WKV.forward(ctx, w, u, k, v)
+
+    @staticmethod
+    def backward(ctx, gy):
+        return (None, None, None) + tuple(WKV.backward(ctx, gy))
+
+
+def RUN_CUDA(*args):
+    """RUN_CUDA(w, u, k, v) (vrwkv.py:64-65) or legacy RUN_CUDA(B, T, C, w, u, k, v)."""
+    if len(args) == 4:
+        w, u, k, v = args
+        return WKV.apply(w.cuda(), u.cuda(), k.cuda(), v.cuda())
+    if len(args) == 7:
+        B, T, C, w, u, k, v = args
+        return _WKVLegacy.apply(B, T, C, w.cuda(), u.cuda(), k.cuda(), v.cuda())
+    raise TypeError("RUN_CUDA takes (w, u, k, v) or (B, T, C, w, u, k, v)")
