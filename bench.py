@@ -17,6 +17,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+# HBM bytes per launch of the fp32 kernel at this shape, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled
+# by a plain device copy of known size (profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md).
+MEASURED_TRAFFIC_FP32 = 115_931_000
 LAYERS = 12
 B, T, C = 64, 196, 768
 
@@ -60,7 +63,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--io", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-calls", type=int, default=4)
+    ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
                          "traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -151,7 +154,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_FP32 if args.io == "fp32" else None,
             "kernel": "biwkv_fwd_kernel (one launch per call)",
             "algorithmic_bytes_per_launch": bytes_alg,
         },
