@@ -17,8 +17,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-# HBM bytes per launch of the fp32 kernel at this shape, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled
-# by a plain device copy of known size (profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md).
+# HBM bytes per launch of the fp32 kernel at this shape: rocprofv3 FETCH_SIZE + WRITE_SIZE of this
+# command with --calibrate-copy, each scaled by what it reads for that plain copy of known size.
 MEASURED_TRAFFIC_FP32 = 115_931_000
 LAYERS = 12
 B, T, C = 64, 196, 768
@@ -69,8 +69,8 @@ def main():
                          "traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (every sequence is independent; see "
-              "DESIGN.md for how the path would shard); use --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (every (batch, channel) sequence is "
+              "independent, so more GPUs would simply split the batch); use --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
