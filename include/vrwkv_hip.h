@@ -51,6 +51,21 @@ int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v
                     int B, int T, int C, int io_dtype,
                     void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* ---- wkv6 forward (bidirectional RWKV-6 scan) -----------------------------------------
+ * Replaces forward(B,T,C,H,r,k,v,w,u,y)
+ *   (classification/mmcls_custom/models/backbones/cuda_v6/wkv6_op.cpp:7-9, launcher
+ *    .../cuda_v6/wkv6_cuda.cu:348-353, kernel :6-97).
+ * r, k, v: (B,T,C) of rkv_dtype; w: (B,T,C) of w_dtype (fp32, or the dtype of r, k, v);
+ * u: (H,64) fp32; y: (B,T,C) fp32, caller-allocated, fully overwritten.  C must be H*64.
+ * w_is_ew = 0: w is the raw decay logit and the kernel uses d = exp(-exp(w)), i.e. it folds in
+ *              the `ew = -exp(w)` of WKV_6.forward (vrwkv6.py:48);
+ * w_is_ew = 1: w already holds ew = -exp(w_raw), as the reference extension receives it.
+ * State and accumulation are fp32.  No limit on T. */
+size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H);
+int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, const float* u,
+                   float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
+                   void* workspace, size_t workspace_bytes, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,8 +1,9 @@
 """MI355X-native WKV operators for Vision-RWKV behind the reference's operator interface.
 
     from vision_rwkv_amd import RUN_CUDA            # Bi-WKV  (VRWKV)
+    from vision_rwkv_amd import RUN_CUDA_RWKV6      # wkv6    (VRWKV6)
 """
 from ._lib import VrwkvError, LIB_PATH, build, lib
-from .ops import WKV, RUN_CUDA, bi_wkv_forward
+from .ops import WKV, RUN_CUDA, bi_wkv_forward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, HEAD_SIZE
 
-__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "VrwkvError", "LIB_PATH", "build", "lib"]
+__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "HEAD_SIZE", "VrwkvError", "LIB_PATH", "build", "lib"]

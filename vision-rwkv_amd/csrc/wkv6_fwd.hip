@@ -1,0 +1,90 @@
+// wkv6 forward entry points.
+#include "wkv6_fwd_scalar.h"
+
+using namespace vrwkv;
+using namespace vrwkv::wkv6_detail;
+
+namespace {
+
+int validate(int B, int T, int C, int H, int rkv_dtype, int w_dtype) {
+    if (B <= 0 || T <= 0 || C <= 0 || H <= 0) {
+        set_error("wkv6_fwd: B, T, C, H must be positive (got %d, %d, %d, %d)", B, T, C, H);
+        return VRWKV_INVALID_ARG;
+    }
+    if (C != H * N) {                                   // assert(H*_N_ == C), wkv6_cuda.cu:350
+        set_error("wkv6_fwd: C must equal H*64 (got C=%d, H=%d)", C, H);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    for (int dt : {rkv_dtype, w_dtype})
+        if (dt != VRWKV_F32 && dt != VRWKV_BF16 && dt != VRWKV_F16) {
+            set_error("wkv6_fwd: unsupported dtype code %d", dt);
+            return VRWKV_UNSUPPORTED_DTYPE;
+        }
+    if (w_dtype != VRWKV_F32 && w_dtype != rkv_dtype) {
+        set_error("wkv6_fwd: w must be fp32 or have the dtype of r, k, v");
+        return VRWKV_UNSUPPORTED_DTYPE;
+    }
+    if ((long long)B * T * C >= (1LL << 40) || (long long)B * H > 0x7fffffffLL) {
+        set_error("wkv6_fwd: tensor too large");
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    return VRWKV_OK;
+}
+
+template <typename IO, typename WT>
+int launch_scalar(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
+                  const unsigned char* todo, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
+    const dim3 grid(B * H), block(256);
+    const IO* rr = static_cast<const IO*>(r);
+    const IO* kk = static_cast<const IO*>(k);
+    const IO* vv = static_cast<const IO*>(v);
+    const WT* ww = static_cast<const WT*>(w);
+    if (w_is_ew) {
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+    } else {
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+    }
+    return check_launch("wkv6_fwd");
+}
+
+}  // namespace
+
+extern "C" size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H) {
+    (void)B; (void)T; (void)C; (void)H;
+    return 0;
+}
+
+extern "C" int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, const float* u,
+                              float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
+                              void* workspace, size_t workspace_bytes, void* hip_stream) {
+    (void)workspace; (void)workspace_bytes;
+    int rc = validate(B, T, C, H, rkv_dtype, w_dtype);
+    if (rc != VRWKV_OK) return rc;
+    if (!r || !k || !v || !w || !u || !y) {
+        set_error("wkv6_fwd: null pointer argument");
+        return VRWKV_INVALID_ARG;
+    }
+    const size_t esz = rkv_dtype == VRWKV_F32 ? 4 : 2, wsz = w_dtype == VRWKV_F32 ? 4 : 2;
+    if ((((uintptr_t)r | (uintptr_t)k | (uintptr_t)v) & (esz - 1)) || ((uintptr_t)w & (wsz - 1)) ||
+        (((uintptr_t)u | (uintptr_t)y) & 3)) {
+        set_error("wkv6_fwd: pointers must be aligned to their element size");
+        return VRWKV_INVALID_ARG;
+    }
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    const bool ew = w_is_ew != 0;
+    switch (rkv_dtype) {
+        case VRWKV_F32:
+            return launch_scalar<float, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+        case VRWKV_BF16:
+            return w_dtype == VRWKV_F32
+                       ? launch_scalar<__hip_bfloat16, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st)
+                       : launch_scalar<__hip_bfloat16, __hip_bfloat16>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+        case VRWKV_F16:
+            return w_dtype == VRWKV_F32
+                       ? launch_scalar<__half, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st)
+                       : launch_scalar<__half, __half>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+    }
+    return VRWKV_UNSUPPORTED_DTYPE;
+}

@@ -4,6 +4,7 @@ libvrwkv_hip.so.
 Mirrors
   WKV / RUN_CUDA(w,u,k,v)                 classification/mmcls_custom/models/backbones/vrwkv.py:29-65
   legacy RUN_CUDA(B,T,C,w,u,k,v)          classification/mae/vrwkv/vrwkv.py:30-90
+  WKV_6 / RUN_CUDA_RWKV6(B,T,C,H,r,k,v,w,u)  classification/mmcls_custom/models/backbones/vrwkv6.py:34-73
 with the same argument meaning, output dtype rule and error behaviour (RuntimeError for
 non-device / non-contiguous tensors).
 """
@@ -99,3 +100,64 @@ def RUN_CUDA(*args):
         B, T, C, w, u, k, v = args
         return _WKVLegacy.apply(B, T, C, w.cuda(), u.cuda(), k.cuda(), v.cuda())
     raise TypeError("RUN_CUDA takes (w, u, k, v) or (B, T, C, w, u, k, v)")
+
+
+HEAD_SIZE = 64   # vrwkv6.py:23
+
+
+def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False):
+    """Extension-level entry (wkv6_op.cpp:7-9): r,k,v (B,T,C) fp32/bf16/fp16, w (B,T,C) fp32 or
+    that dtype, u (H,64); returns y (B,T,C) fp32.  With w_is_ew=False, w is the raw decay logit
+    (the kernel applies d = exp(-exp(w))); with True it is ew = -exp(w_raw) as the reference
+    extension receives it."""
+    for t, n in ((r, "r"), (k, "k"), (v, "v"), (w, "w"), (u, "u")):
+        _check_input(t, n)
+    if tuple(r.shape) != (B, T, C) or k.shape != r.shape or v.shape != r.shape or w.shape != r.shape:
+        raise RuntimeError("r, k, v, w must all be (B,T,C)")
+    if u.numel() != C:
+        raise RuntimeError("u must have H*64 = C elements")
+    if r.dtype not in _DT or k.dtype != r.dtype or v.dtype != r.dtype:
+        raise RuntimeError("r, k, v must share one of float32 / bfloat16 / float16")
+    if w.dtype != torch.float32 and w.dtype != r.dtype:
+        raise RuntimeError("w must be float32 or have the dtype of r, k, v")
+    uf = u if u.dtype == torch.float32 else u.float()
+    L = _lib.lib()
+    y = torch.empty((B, T, C), device=r.device, dtype=torch.float32)
+    if y.numel() == 0:
+        return y
+    ws_bytes = L.vrwkv_wkv6_fwd_workspace_bytes(B, T, C, H)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device) if ws_bytes else None
+    with torch.cuda.device(r.device):
+        _lib.check(L.vrwkv_wkv6_fwd(r.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), uf.data_ptr(),
+                                    y.data_ptr(), B, T, C, H, _DT[r.dtype], _DT[w.dtype], 1 if w_is_ew else 0,
+                                    ws.data_ptr() if ws is not None else None, ws_bytes,
+                                    _stream_ptr(r.device)))
+    return y
+
+
+class WKV_6(torch.autograd.Function):
+    """Bidirectional RWKV-6 scan with the reference's call contract (vrwkv6.py:34-70): contiguous
+    (B,T,C) inputs, raw decay logit w, fp32 (B,T,C) result.  The `ew = -exp(w)` tensor the
+    reference materialises is folded into the kernel."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u):
+        with torch.no_grad():
+            assert HEAD_SIZE == C // H
+            ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            assert r.is_contiguous()
+            assert k.is_contiguous()
+            assert v.is_contiguous()
+            assert w.is_contiguous()
+            assert u.is_contiguous()
+            ctx.save_for_backward(r, k, v, w, u)
+            return wkv6_forward(B, T, C, H, r, k, v, w, u)
+
+    @staticmethod
+    def backward(ctx, gy):
+        raise NotImplementedError("wkv6 backward is not built yet in this library")
+
+
+def RUN_CUDA_RWKV6(B, T, C, H, r, k, v, w, u):
+    """vrwkv6.py:72-73."""
+    return WKV_6.apply(B, T, C, H, r, k, v, w, u)
