@@ -80,6 +80,25 @@ def test_extreme_decay(ops, w_mean):
     assert rel_err(y, clib.wkv6_fwd(r, k, v, w, u, 2)) <= TOL
 
 
+def test_chunked_and_sequential_kernels_agree(ops, monkeypatch):
+    """The matrix-core path and the sequential-state path are independent implementations."""
+    r, k, v, w, u = gen(3, 196, 2, 21)
+    y_chunk, *_ = run(ops, r, k, v, w, u, 2, torch.bfloat16)
+    monkeypatch.setenv("VRWKV_WKV6_PATH", "scalar")
+    y_seq, *_ = run(ops, r, k, v, w, u, 2, torch.bfloat16)
+    assert rel_err(y_chunk, y_seq) <= TOL
+
+
+def test_mixed_ranges_fall_back_per_sequence(ops):
+    """One head with a decay far outside the chunked kernel's range, the other ordinary."""
+    from oracle import clib
+    r, k, v, w, u = gen(2, 130, 2, 31)
+    w[:, :, :64] = 3.0 + 0.2 * w[:, :, :64]
+    y, *_ = run(ops, r, k, v, w, u, 2)
+    assert np.isfinite(y).all()
+    assert rel_err(y, clib.wkv6_fwd(r, k, v, w, u, 2)) <= TOL
+
+
 def test_reversal_and_head_independence(ops):
     r, k, v, w, u = gen(2, 50, 2, 5)
     y, *_ = run(ops, r, k, v, w, u, 2)

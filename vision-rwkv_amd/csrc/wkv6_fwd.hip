@@ -1,5 +1,8 @@
 // wkv6 forward entry points.
 #include "wkv6_fwd_scalar.h"
+#include "wkv6_fwd_chunk.h"
+#include <cstdlib>
+#include <cstring>
 
 using namespace vrwkv;
 using namespace vrwkv::wkv6_detail;
@@ -49,19 +52,58 @@ int launch_scalar(const void* r, const void* k, const void* v, const void* w, co
     return check_launch("wkv6_fwd");
 }
 
+// Chunked matrix-core passes (descending, then ascending), then the exact kernel for whatever
+// sequences they flagged as out of range.
+template <typename IO, typename WT>
+int launch_chunked(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
+                   unsigned char* todo, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
+    const dim3 grid(B * H), block(128);
+    const IO* rr = static_cast<const IO*>(r);
+    const IO* kk = static_cast<const IO*>(k);
+    const IO* vv = static_cast<const IO*>(v);
+    const WT* ww = static_cast<const WT*>(w);
+    if (w_is_ew) {
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 1, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 0, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+    } else {
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 1, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 0, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+    }
+    const int rc = check_launch("wkv6_fwd (chunked)");
+    if (rc != VRWKV_OK) return rc;
+    return launch_scalar<IO, WT>(r, k, v, w, u, y, todo, B, T, C, H, w_is_ew, st);
+}
+
+bool force_scalar() {
+    const char* s = getenv("VRWKV_WKV6_PATH");           // tuning / testing override
+    return s && !strcmp(s, "scalar");
+}
+
+template <typename IO, typename WT>
+int launch_any(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
+               void* ws, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
+    if (force_scalar()) return launch_scalar<IO, WT>(r, k, v, w, u, y, nullptr, B, T, C, H, w_is_ew, st);
+    return launch_chunked<IO, WT>(r, k, v, w, u, y, static_cast<unsigned char*>(ws), B, T, C, H, w_is_ew, st);
+}
+
 }  // namespace
 
 extern "C" size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H) {
-    (void)B; (void)T; (void)C; (void)H;
-    return 0;
+    (void)T; (void)C;
+    if (B <= 0 || H <= 0) return 0;
+    return ((size_t)2 * B * H + 255) & ~(size_t)255;     // one "left to the exact kernel" flag per pass and sequence
 }
 
 extern "C" int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, const float* u,
                               float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
                               void* workspace, size_t workspace_bytes, void* hip_stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = validate(B, T, C, H, rkv_dtype, w_dtype);
     if (rc != VRWKV_OK) return rc;
+    if (!force_scalar() && (!workspace || workspace_bytes < (size_t)2 * B * H)) {
+        set_error("wkv6_fwd: workspace of %zu bytes required (got %zu)", (size_t)2 * B * H,
+                  workspace ? workspace_bytes : (size_t)0);
+        return VRWKV_WORKSPACE_TOO_SMALL;
+    }
     if (!r || !k || !v || !w || !u || !y) {
         set_error("wkv6_fwd: null pointer argument");
         return VRWKV_INVALID_ARG;
@@ -76,15 +118,15 @@ extern "C" int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const
     const bool ew = w_is_ew != 0;
     switch (rkv_dtype) {
         case VRWKV_F32:
-            return launch_scalar<float, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+            return launch_any<float, float>(r, k, v, w, u, y, workspace, B, T, C, H, ew, st);
         case VRWKV_BF16:
             return w_dtype == VRWKV_F32
-                       ? launch_scalar<__hip_bfloat16, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st)
-                       : launch_scalar<__hip_bfloat16, __hip_bfloat16>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+                       ? launch_any<__hip_bfloat16, float>(r, k, v, w, u, y, workspace, B, T, C, H, ew, st)
+                       : launch_any<__hip_bfloat16, __hip_bfloat16>(r, k, v, w, u, y, workspace, B, T, C, H, ew, st);
         case VRWKV_F16:
             return w_dtype == VRWKV_F32
-                       ? launch_scalar<__half, float>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st)
-                       : launch_scalar<__half, __half>(r, k, v, w, u, y, nullptr, B, T, C, H, ew, st);
+                       ? launch_any<__half, float>(r, k, v, w, u, y, workspace, B, T, C, H, ew, st)
+                       : launch_any<__half, __half>(r, k, v, w, u, y, workspace, B, T, C, H, ew, st);
     }
     return VRWKV_UNSUPPORTED_DTYPE;
 }

@@ -25,7 +25,8 @@ void wkv6_fwd_scalar_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_
                             const WT* __restrict__ w_, const float* __restrict__ u_, float* __restrict__ y_,
                             const unsigned char* __restrict__ todo, int T, int C, int H)
 {
-    if (todo && !todo[blockIdx.x]) return;               // (b,h) already done by the chunked kernel
+    // `todo` (one flag per pass and sequence) marks what the chunked kernel left undone
+    if (todo && !(todo[blockIdx.x] | todo[gridDim.x + blockIdx.x])) return;
     __shared__ __attribute__((aligned(16))) float s_row[4][2][3][N];   // [wave][buffer][r,k,d][j]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
