@@ -28,6 +28,7 @@
 // kernel: the pass records it in `todo` and stops.
 #pragma once
 #include "vrwkv_common.h"
+#include <type_traits>
 
 namespace vrwkv {
 namespace wkv6_detail {
@@ -46,10 +47,19 @@ constexpr float SAFE_DECAY = 60.f;
 __device__ __forceinline__ bf16x8 cat8(bf16x4 a, bf16x4 b) {
     return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
+// Sum over the 64 lanes, result wave-uniform: four DPP steps inside each 16-lane row (VALU rate),
+// then the four row sums through scalar registers.
 __device__ __forceinline__ float wave_sum(float x) {
-    x += __shfl_xor(x, 32); x += __shfl_xor(x, 16); x += __shfl_xor(x, 8);
-    x += __shfl_xor(x, 4);  x += __shfl_xor(x, 2);  x += __shfl_xor(x, 1);
-    return x;
+    auto dpp = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
+    };
+    x += dpp(x, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
+    x += dpp(x, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
+    x += dpp(x, std::integral_constant<int, 0x141>{});   // row_half_mirror
+    x += dpp(x, std::integral_constant<int, 0x140>{});   // row_mirror
+    const int xi = __builtin_bit_cast(int, x);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
 }
 // head/tail split of eight fp32 accumulator values into two packed bf16 operands
 __device__ __forceinline__ void split8(const float (&x)[8], bf16x8& hi, bf16x8& lo) {
