@@ -56,6 +56,51 @@ def cpu_baseline(torch, n_calls):
     }, y
 
 
+def wkv6_section(torch, ops, steps, warmup, with_cpu):
+    """Secondary line of the metric: wkv6 forward at the VRWKV6-B shape (B=64, T=196, C=768, H=12,
+    bf16 r,k,v, fp32 w and y).  tokens/s = B*T per call; MFMA figures use the flops the chunked
+    kernel issues to the matrix cores (all split-bf16 products counted), end to end."""
+    Bw, Tw, Hw = 64, 196, 12
+    Cw = Hw * 64
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(4321)
+    r, k, v = (torch.randn(Bw, Tw, Cw, generator=g).to(dev).bfloat16() for _ in range(3))
+    w = (torch.randn(Bw, Tw, Cw, generator=g) * 0.5 - 0.5).to(dev)
+    u = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
+    for _ in range(warmup):
+        ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        y = ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / steps
+    nchunk = (Tw + 31) // 32
+    # per chunk, pass and value half (one wave): 36 MFMA 32x32x16 = 36 * 32768 flop
+    mfma_flops = Bw * Hw * 2 * nchunk * 2 * 36 * 32768
+    out = {
+        "workload": f"wkv6 forward B={Bw} T={Tw} C={Cw} H={Hw}, bf16 r,k,v, fp32 w,y",
+        "us_per_call": round(us, 2),
+        "tokens_per_s": round(Bw * Tw / (us * 1e-6), 1),
+        "recurrence_tflops": round(Bw * Tw * Hw * (10 * 64 * 64 + 3 * 64) / (us * 1e-6) / 1e12, 2),
+        "mfma_issued_tflops": round(mfma_flops / (us * 1e-6) / 1e12, 2),
+        "pct_bf16_mfma_peak_end_to_end": round(100.0 * mfma_flops / (us * 1e-6) / 2.5e15, 3),
+    }
+    if with_cpu:
+        from oracle import torch_eager
+        bs = 4
+        rc, kc, vc, wc = (t[:bs].float().cpu() for t in (r, k, v, w))
+        t0 = time.perf_counter()
+        torch_eager.wkv6_eager(rc, kc, vc, wc, u.cpu(), Hw)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(bs * Tw / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"{bs} of the {Bw} batch elements, PyTorch CPU eager "
+                                                         f"two-pass recurrence, {dt:.1f} s"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -63,6 +108,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--io", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-wkv6", action="store_true", help="skip the secondary wkv6 measurement")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -130,7 +176,7 @@ def main():
     gbs = bytes_alg / (us_per_launch * 1e-6) / 1e9
 
     out = {
-        "metric": "Bi-WKV fwd GB/s (% HBM peak) @VRWKV-B",
+        "metric": "Bi-WKV fwd GB/s (% HBM peak) @VRWKV-B; wkv6 tokens/s (% MFMA peak)",
         "value": round(gbs, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -162,6 +208,8 @@ def main():
     if not args.no_cpu_baseline:
         cb, y_cpu = cpu_baseline(torch, args.cpu_calls)
         out["cpu_baseline"] = cb
+    if not args.no_wkv6:
+        out["wkv6"] = wkv6_section(torch, ops, max(args.steps, 10), max(args.warmup // 5, 3), not args.no_cpu_baseline)
     print(json.dumps(out))
 
 
