@@ -6,10 +6,10 @@
 // classification/mmcls_custom/models/backbones/cuda_new/bi_wkv_kernel.cu:93-108.
 //
 // Work decomposition (nothing like the reference's 32 token-chunks x 32 channels block):
-//   lane      = VEC adjacent channels  -> every load/store instruction of a wave touches
-//               one contiguous 64*VEC-element row segment of k, v or y;
+//   lane      = one channel -> every load/store instruction of a wave touches one contiguous
+//               64-channel row segment of k, v or y;
 //   wave      = L consecutive tokens of those channels, held in registers;
-//   workgroup = S waves = S*L consecutive tokens (a "super-chunk") of 64*VEC channels;
+//   workgroup = S <= 8 waves = S*L consecutive tokens (a "super-chunk") of 64 channels;
 //   tile      = (batch, super-chunk, channel tile); workgroups are persistent and walk the
 //               tiles with stride gridDim.x, loading tile n+1 into a second register set
 //               while tile n is being computed, so HBM traffic overlaps the arithmetic.
@@ -19,21 +19,23 @@
 // main kernel read the tokens a second time.
 // All tensor accesses are raw buffer loads/stores on a per-batch-element descriptor, so
 // tokens past T and channels past C are dropped by the hardware range check instead of
-// by exec-mask branches.
+// by exec-mask branches; the streamed tensors use the non-temporal cache policy.
 //
 // Arithmetic is in the log2 domain (kappa = k*log2e, omega = w*log2e, mu = u*log2e) so
 // that every exponential is one v_exp_f32.
 //
 // Two code paths, chosen per tile from (w, u, T) alone and therefore identically by
 // every wave that touches a channel tile:
-//   fast   |omega|*(T+1) + |mu| <= 40.  One reference exponent R = max_t kappa_t per
-//          sequence; E_t = 2^(kappa_t-R) <= 1 is computed once per token and reused by
-//          both directions and both phases; states are plain decayed sums
-//          a <- g*a + E_t v_t (g = 2^-omega), no per-token max.  Under the bound every
-//          state stays within 2^+-41 of the largest term, so nothing overflows, and a
+//   fast   |omega|*(T+1) + |mu| <= 40.  Each wave uses its own integer reference exponent
+//          Rw = ceil(max kappa) over its tokens; E_t = 2^(kappa_t-Rw) <= 1 is computed once per
+//          token and reused by both directions and both phases; states are plain decayed sums
+//          a <- g*a + E_t v_t (g = 2^-omega), no per-token max.  Waves exchange their chunk
+//          aggregates once per tile and rescale each other's by exact powers of two.  Under the
+//          bound every state stays within 2^+-41 of the largest term, so nothing overflows, and a
 //          term that underflows is below 2^-80 of its denominator.
 //   robust anything else: every state is a (num, den, exponent) triple renormalised at
-//          every token, exactly the reference's recurrence, for both directions.
+//          every token, exactly the reference's recurrence, for both directions; those tiles
+//          are done in a second walk after the fast ones.
 #pragma once
 #include "vrwkv_common.h"
 
