@@ -51,6 +51,19 @@ int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v
                     int B, int T, int C, int io_dtype,
                     void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* ---- Bi-WKV backward ------------------------------------------------------------------
+ * Replaces bi_wkv_backward(w,u,k,v,gy) -> [gw,gu,gk,gv]
+ *   (classification/mmcls_custom/models/backbones/cuda_new/bi_wkv.cpp:35-47, launcher
+ *    .../cuda_new/bi_wkv_kernel.cu:401-443, kernel :119-367) and the legacy
+ *   backward(B,T,C,w,u,k,v,gy,gw,gu,gk,gv) (.../backbones/cuda/wkv_op.cpp:9-11).
+ * w, u, gw, gu: (C,) fp32, gw and gu already summed over batch and tokens (fully overwritten,
+ * no need to zero them); k, v, gy, gk, gv: (B,T,C) of io_dtype.  The workspace (always needed)
+ * replaces the three scratch tensors the reference allocates (bi_wkv_kernel.cu:415-417). */
+size_t vrwkv_biwkv_bwd_workspace_bytes(int B, int T, int C, int io_dtype);
+int vrwkv_biwkv_bwd(const float* w, const float* u, const void* k, const void* v, const void* gy,
+                    float* gw, float* gu, void* gk, void* gv, int B, int T, int C, int io_dtype,
+                    void* workspace, size_t workspace_bytes, void* hip_stream);
+
 /* ---- wkv6 forward (bidirectional RWKV-6 scan) -----------------------------------------
  * Replaces forward(B,T,C,H,r,k,v,w,u,y)
  *   (classification/mmcls_custom/models/backbones/cuda_v6/wkv6_op.cpp:7-9, launcher

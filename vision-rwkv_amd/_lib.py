@@ -47,6 +47,10 @@ def _declare(lib):
     lib.vrwkv_biwkv_fwd_workspace_bytes.restype = sz
     lib.vrwkv_biwkv_fwd.argtypes = [fp, fp, vp, vp, vp, i, i, i, i, vp, sz, vp]
     lib.vrwkv_biwkv_fwd.restype = i
+    lib.vrwkv_biwkv_bwd_workspace_bytes.argtypes = [i, i, i, i]
+    lib.vrwkv_biwkv_bwd_workspace_bytes.restype = sz
+    lib.vrwkv_biwkv_bwd.argtypes = [fp, fp, vp, vp, vp, fp, fp, vp, vp, i, i, i, i, vp, sz, vp]
+    lib.vrwkv_biwkv_bwd.restype = i
     lib.vrwkv_wkv6_fwd_workspace_bytes.argtypes = [i, i, i, i]
     lib.vrwkv_wkv6_fwd_workspace_bytes.restype = sz
     lib.vrwkv_wkv6_fwd.argtypes = [vp, vp, vp, vp, fp, vp, i, i, i, i, i, i, i, vp, sz, vp]

@@ -55,6 +55,36 @@ def bi_wkv_forward(w, u, k, v):
     return y
 
 
+def bi_wkv_backward(w, u, k, v, gy):
+    """Extension-level entry (bi_wkv.cpp:35-47): w,u (C,) fp32; k,v,gy (B,T,C) of one dtype;
+    returns [gw, gu, gk, gv] with gw, gu (C,) fp32 summed over batch and tokens and gk, gv of the
+    dtype of k."""
+    for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v"), (gy, "gy")):
+        _check_input(t, n)
+    if k.dim() != 3 or v.shape != k.shape or gy.shape != k.shape:
+        raise RuntimeError("k, v and gy must all be (B,T,C)")
+    B, T, C = k.shape
+    if w.numel() != C or u.numel() != C or w.dtype != torch.float32 or u.dtype != torch.float32:
+        raise RuntimeError("w and u must be float32 with C elements")
+    if k.dtype not in _DT or v.dtype != k.dtype or gy.dtype != k.dtype:
+        raise RuntimeError("k, v and gy must share one of float32 / bfloat16 / float16")
+    L = _lib.lib()
+    dt = _DT[k.dtype]
+    gw = torch.empty(C, dtype=torch.float32, device=k.device)
+    gu = torch.empty(C, dtype=torch.float32, device=k.device)
+    gk = torch.empty_like(k)
+    gv = torch.empty_like(k)
+    if k.numel() == 0:
+        return [gw.zero_(), gu.zero_(), gk, gv]
+    ws_bytes = L.vrwkv_biwkv_bwd_workspace_bytes(B, T, C, dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=k.device)
+    with torch.cuda.device(k.device):
+        _lib.check(L.vrwkv_biwkv_bwd(w.data_ptr(), u.data_ptr(), k.data_ptr(), v.data_ptr(), gy.data_ptr(),
+                                     gw.data_ptr(), gu.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                                     B, T, C, dt, ws.data_ptr(), ws_bytes, _stream_ptr(k.device)))
+    return [gw, gu, gk, gv]
+
+
 class WKV(torch.autograd.Function):
     """Bi-WKV with the reference's dtype rule: arithmetic in fp32, the result is fp32 unless
     the *parameter* w is half / bfloat16, in which case it has w's dtype (vrwkv.py:31-44).
@@ -74,7 +104,19 @@ class WKV(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy):
-        raise NotImplementedError("Bi-WKV backward is not built yet in this library")
+        # vrwkv.py:47-61: gradients in fp32, returned in w's dtype when that is half / bfloat16
+        w, u, k, v = ctx.saved_tensors
+        out_dtype = w.dtype if w.dtype in (torch.half, torch.bfloat16) else torch.float32
+        wf = w.float().contiguous()
+        uf = u.float().contiguous()
+        if k.dtype == out_dtype and v.dtype == out_dtype and out_dtype != torch.float32:
+            gw, gu, gk, gv = bi_wkv_backward(wf, uf, k.contiguous(), v.contiguous(), gy.to(out_dtype).contiguous())
+        else:
+            gw, gu, gk, gv = bi_wkv_backward(wf, uf, k.float().contiguous(), v.float().contiguous(),
+                                             gy.float().contiguous())
+        if out_dtype == torch.float32:
+            return (gw, gu, gk, gv)
+        return (gw.to(out_dtype), gu.to(out_dtype), gk.to(out_dtype), gv.to(out_dtype))
 
 
 class _WKVLegacy(torch.autograd.Function):
