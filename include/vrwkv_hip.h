@@ -79,6 +79,19 @@ int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, c
                    float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
                    void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* ---- wkv6 backward ---------------------------------------------------------------------
+ * Replaces backward(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu)
+ *   (classification/mmcls_custom/models/backbones/cuda_v6/wkv6_op.cpp:10-12, launcher
+ *    .../cuda_v6/wkv6_cuda.cu:355-362, kernels :99-346), without its T <= 256 limit.
+ * r, k, v, w, u as in vrwkv_wkv6_fwd; gy, gr, gk, gv, gw: (B,T,C) fp32, fully overwritten; gw is the
+ * gradient w.r.t. the raw decay logit (wkv6_cuda.cu:248,277); gu: (H,64) fp32 already summed over
+ * the batch (the reference returns (B,C) and sums in Python, vrwkv6.py:69). */
+size_t vrwkv_wkv6_bwd_workspace_bytes(int B, int T, int C, int H);
+int vrwkv_wkv6_bwd(const void* r, const void* k, const void* v, const void* w, const float* u,
+                   const float* gy, float* gr, float* gk, float* gv, float* gw, float* gu,
+                   int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
+                   void* workspace, size_t workspace_bytes, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

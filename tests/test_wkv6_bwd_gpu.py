@@ -1,0 +1,70 @@
+"""Parity of the HIP wkv6 backward with autograd through the float64 closed form.
+Tolerance: err = max|g - ref| / max(|ref|, rms(ref)) <= 1e-3."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_golden, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import vision_rwkv_amd
+    assert torch.cuda.is_available()
+    return vision_rwkv_amd
+
+
+def run(ops, r, k, v, w, u, gy, H, dtype=torch.float32):
+    dev = "cuda:0"
+    t = lambda a, d=torch.float32: torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(dev).to(d)
+    rt, kt, vt = t(r, dtype), t(k, dtype), t(v, dtype)
+    B, T, C = rt.shape
+    out = ops.wkv6_backward(B, T, C, H, rt, kt, vt, t(w), t(u), t(gy))
+    torch.cuda.synchronize()
+    f = lambda x: x.float().cpu().numpy()
+    return [f(x) for x in out], f(rt), f(kt), f(vt)
+
+
+def test_golden_gradient_fixture(ops):
+    g = load_golden("wkv6_golden")["grad_T9"]
+    (gr, gk, gv, gw, gu), *_ = run(ops, g["r"], g["k"], g["v"], g["w"], g["u"], g["gy"], 1)
+    for got, name in ((gr, "gr"), (gk, "gk"), (gv, "gv"), (gw, "gw"), (gu, "gu")):
+        assert rel_err(got, g[name]) <= TOL, name
+
+
+@pytest.mark.parametrize("B,T,H,w_mean", [(1, 1, 1, -0.5), (2, 5, 2, -0.5), (2, 40, 1, -0.5), (1, 300, 1, -3.0), (1, 30, 1, 1.0)])
+def test_against_autograd_closed_form(ops, B, T, H, w_mean):
+    from oracle import wkv6
+    rng = np.random.default_rng(T * 7 + H)
+    C = H * 64
+    r, k, v, gy = (rng.standard_normal((B, T, C)).astype(np.float32) for _ in range(4))
+    w = rng.normal(w_mean, 0.5, (B, T, C)).astype(np.float32)
+    u = rng.normal(0, 0.1, (H, 64)).astype(np.float32)
+    (gr, gk, gv, gw, gu), *_ = run(ops, r, k, v, w, u, gy, H)
+    ref = wkv6.wkv6_grads_closed(r, k, v, w, u, H, gy)
+    for got, want, name in zip((gr, gk, gv, gw, gu), ref, ("gr", "gk", "gv", "gw", "gu")):
+        if T == 1 and name == "gw":
+            assert np.abs(got).max() <= 1e-6
+            continue
+        assert rel_err(got, want) <= TOL, name
+
+
+def test_bf16_inputs_and_autograd_function(ops):
+    from oracle import wkv6
+    B, T, H = 2, 33, 2
+    C = H * 64
+    g = torch.Generator().manual_seed(8)
+    r, k, v = (torch.randn(B, T, C, generator=g).bfloat16() for _ in range(3))
+    w = torch.randn(B, T, C, generator=g) * 0.5 - 0.5
+    u = torch.randn(H, 64, generator=g) * 0.1
+    gy = torch.randn(B, T, C, generator=g)
+    leaves = [t.cuda().requires_grad_(True) for t in (r, k, v, w, u)]
+    y = ops.RUN_CUDA_RWKV6(B, T, C, H, *leaves)
+    y.backward(gy.cuda())
+    ref = wkv6.wkv6_grads_closed(r.float().numpy(), k.float().numpy(), v.float().numpy(), w.numpy(), u.numpy(), H, gy.numpy())
+    for leaf, want, tol in zip(leaves, ref, (1e-2, 1e-2, 1e-2, TOL, TOL)):   # r,k,v grads come back in bf16
+        assert rel_err(leaf.grad.float().cpu().numpy(), want) <= tol
+    assert tuple(leaves[4].grad.shape) == (H, 64)

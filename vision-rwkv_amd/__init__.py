@@ -4,6 +4,6 @@
     from vision_rwkv_amd import RUN_CUDA_RWKV6      # wkv6    (VRWKV6)
 """
 from ._lib import VrwkvError, LIB_PATH, build, lib
-from .ops import WKV, RUN_CUDA, bi_wkv_forward, bi_wkv_backward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, HEAD_SIZE
+from .ops import WKV, RUN_CUDA, bi_wkv_forward, bi_wkv_backward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, wkv6_backward, HEAD_SIZE
 
-__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "HEAD_SIZE", "VrwkvError", "LIB_PATH", "build", "lib"]
+__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "wkv6_backward", "HEAD_SIZE", "VrwkvError", "LIB_PATH", "build", "lib"]

@@ -177,6 +177,35 @@ def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False):
     return y
 
 
+def wkv6_backward(B, T, C, H, r, k, v, w, u, gy, w_is_ew=False):
+    """Extension-level entry (wkv6_op.cpp:10-12): returns (gr, gk, gv, gw) as (B,T,C) fp32 and gu as
+    (H,64) fp32 (already summed over the batch); gw is the gradient w.r.t. the raw decay logit."""
+    for t, n in ((r, "r"), (k, "k"), (v, "v"), (w, "w"), (u, "u"), (gy, "gy")):
+        _check_input(t, n)
+    if tuple(r.shape) != (B, T, C) or any(x.shape != r.shape for x in (k, v, w, gy)):
+        raise RuntimeError("r, k, v, w, gy must all be (B,T,C)")
+    if r.dtype not in _DT or k.dtype != r.dtype or v.dtype != r.dtype:
+        raise RuntimeError("r, k, v must share one of float32 / bfloat16 / float16")
+    if w.dtype != torch.float32 and w.dtype != r.dtype:
+        raise RuntimeError("w must be float32 or have the dtype of r, k, v")
+    uf = u if u.dtype == torch.float32 else u.float()
+    gyf = gy if gy.dtype == torch.float32 else gy.float()
+    L = _lib.lib()
+    mk = lambda: torch.empty((B, T, C), device=r.device, dtype=torch.float32)
+    gr, gk, gv, gw = mk(), mk(), mk(), mk()
+    gu = torch.empty((H, C // H), device=r.device, dtype=torch.float32)
+    if gr.numel() == 0:
+        return gr, gk, gv, gw, gu.zero_()
+    ws_bytes = L.vrwkv_wkv6_bwd_workspace_bytes(B, T, C, H)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device)
+    with torch.cuda.device(r.device):
+        _lib.check(L.vrwkv_wkv6_bwd(r.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), uf.data_ptr(),
+                                    gyf.data_ptr(), gr.data_ptr(), gk.data_ptr(), gv.data_ptr(), gw.data_ptr(),
+                                    gu.data_ptr(), B, T, C, H, _DT[r.dtype], _DT[w.dtype], 1 if w_is_ew else 0,
+                                    ws.data_ptr(), ws_bytes, _stream_ptr(r.device)))
+    return gr, gk, gv, gw, gu
+
+
 class WKV_6(torch.autograd.Function):
     """Bidirectional RWKV-6 scan with the reference's call contract (vrwkv6.py:34-70): contiguous
     (B,T,C) inputs, raw decay logit w, fp32 (B,T,C) result.  The `ew = -exp(w)` tensor the
@@ -197,7 +226,12 @@ class WKV_6(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy):
-        raise NotImplementedError("wkv6 backward is not built yet in this library")
+        # vrwkv6.py:55-70: fp32 gradients, gu summed over the batch and shaped (H, C//H)
+        with torch.no_grad():
+            assert gy.is_contiguous()
+            r, k, v, w, u = ctx.saved_tensors
+            gr, gk, gv, gw, gu = wkv6_backward(ctx.B, ctx.T, ctx.C, ctx.H, r, k, v, w, u, gy)
+            return (None, None, None, None, gr, gk, gv, gw, gu)
 
 
 def RUN_CUDA_RWKV6(B, T, C, H, r, k, v, w, u):
