@@ -92,6 +92,18 @@ int vrwkv_wkv6_bwd(const void* r, const void* k, const void* v, const void* w, c
                    int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
                    void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* ---- fused Q-Shift + token mix (the elementwise step in front of the r/k/v projections) -----
+ * Replaces q_shift (classification/mmcls_custom/models/backbones/vrwkv.py:68-79) followed by the
+ * lerps x*mix_m + q_shift(x)*(1-mix_m) of VRWKV_SpatialMix.jit_func (:160-163, n_mix = 3) and
+ * VRWKV_ChannelMix.forward (:248-250, n_mix = 2); with head_dim = 64 the shift is q_shift_multihead
+ * (.../vrwkv6.py:75-100).  The reference has no native code for this step (pure PyTorch ops).
+ * x, out[m]: (B,T,C) of io_dtype; mix: (n_mix, C) fp32; tokens row-major over the (Hp,Wp) patch
+ * grid, T == Hp*Wp or Hp*Wp + 1 (one trailing class token, passed through).
+ * quarter_width = int(C*gamma) (head_dim = 0) or head_dim/4 (per-head quarters). */
+int vrwkv_qshift_mix(const void* x, const float* mix, void* const* out, int n_mix,
+                     int B, int T, int C, int Hp, int Wp, int shift_pixel, int quarter_width,
+                     int head_dim, int io_dtype, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

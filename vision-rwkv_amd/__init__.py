@@ -4,6 +4,8 @@
     from vision_rwkv_amd import RUN_CUDA_RWKV6      # wkv6    (VRWKV6)
 """
 from ._lib import VrwkvError, LIB_PATH, build, lib
-from .ops import WKV, RUN_CUDA, bi_wkv_forward, bi_wkv_backward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, wkv6_backward, HEAD_SIZE
+from .ops import WKV, RUN_CUDA, bi_wkv_forward, bi_wkv_backward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, wkv6_backward, HEAD_SIZE, q_shift, q_shift_mix
 
-__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "wkv6_backward", "HEAD_SIZE", "VrwkvError", "LIB_PATH", "build", "lib"]
+from .backbone import VRWKV, vrwkv_l
+
+__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "wkv6_backward", "HEAD_SIZE", "q_shift", "q_shift_mix", "VRWKV", "vrwkv_l", "VrwkvError", "LIB_PATH", "build", "lib"]

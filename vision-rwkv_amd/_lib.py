@@ -59,6 +59,8 @@ def _declare(lib):
     lib.vrwkv_wkv6_bwd_workspace_bytes.restype = sz
     lib.vrwkv_wkv6_bwd.argtypes = [vp, vp, vp, vp, fp, fp, fp, fp, fp, fp, fp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.vrwkv_wkv6_bwd.restype = i
+    lib.vrwkv_qshift_mix.argtypes = [vp, fp, c.POINTER(c.c_void_p), i, i, i, i, i, i, i, i, i, i, vp]
+    lib.vrwkv_qshift_mix.restype = i
     return lib
 
 

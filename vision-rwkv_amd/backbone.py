@@ -1,0 +1,168 @@
+"""Plain-PyTorch VRWKV backbone (no mmcv / mmcls) that calls the HIP Bi-WKV through RUN_CUDA.
+
+It exists to time the operator in situ (VRWKV-L forward, benchmark config 4) and mirrors, module
+for module and parameter name for parameter name,
+classification/mmcls_custom/models/backbones/vrwkv.py:82-432 (identical copy:
+classification_internimage/models/vrwkv.py) with the VRWKV-L settings of
+classification_internimage/configs/vrwkv_l_22kto1k_384.yaml:10-28.  PatchEmbed is
+Conv2d(kernel = stride = patch) + flatten (mmcv's PatchEmbed with these arguments) and the position
+embedding is resized bicubically as in detection/mmdet_custom/models/utils/embed.py:6-47.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .ops import RUN_CUDA, q_shift, q_shift_mix
+
+
+def resize_pos_embed(pos_embed, src_shape, dst_shape, mode="bicubic"):
+    if tuple(src_shape) == tuple(dst_shape):
+        return pos_embed
+    _, L, C = pos_embed.shape
+    w = pos_embed.reshape(1, src_shape[0], src_shape[1], C).permute(0, 3, 1, 2)
+    w = F.interpolate(w.float(), size=dst_shape, align_corners=False, mode=mode).to(pos_embed.dtype)
+    return torch.flatten(w, 2).transpose(1, 2)
+
+
+def _mix(x, mixes, shift_pixel, gamma, patch_resolution, fused):
+    """[x*m + q_shift(x)*(1-m) for m in mixes]: one fused kernel at inference, tensor ops under autograd."""
+    if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or mixes[0].requires_grad)):
+        return q_shift_mix(x.contiguous(), mixes, shift_pixel, gamma, patch_resolution)
+    xx = q_shift(x, shift_pixel, gamma, patch_resolution)
+    return [x * m + xx * (1 - m) for m in mixes]
+
+
+class VRWKV_SpatialMix(nn.Module):
+    def __init__(self, n_embd, n_layer, layer_id, channel_gamma=1 / 4, shift_pixel=1, key_norm=False, fused_shift=True):
+        super().__init__()
+        self.layer_id, self.n_layer, self.n_embd = layer_id, n_layer, n_embd
+        self.shift_pixel, self.channel_gamma, self.fused_shift = shift_pixel, channel_gamma, fused_shift
+        r01 = layer_id / max(n_layer - 1, 1)
+        r10 = 1.0 - layer_id / n_layer
+        h = torch.arange(n_embd, dtype=torch.float32)
+        self.spatial_decay = nn.Parameter(-5 + 8 * (h / (n_embd - 1)) ** (0.7 + 1.3 * r01))
+        zigzag = torch.tensor([(i + 1) % 3 - 1 for i in range(n_embd)], dtype=torch.float32) * 0.5
+        self.spatial_first = nn.Parameter(torch.ones(n_embd) * math.log(0.3) + zigzag)
+        x = (h / n_embd).reshape(1, 1, n_embd)
+        self.spatial_mix_k = nn.Parameter(torch.pow(x, r10))
+        self.spatial_mix_v = nn.Parameter(torch.pow(x, r10) + 0.3 * r01)
+        self.spatial_mix_r = nn.Parameter(torch.pow(x, 0.5 * r10))
+        self.key = nn.Linear(n_embd, n_embd, bias=False)
+        self.value = nn.Linear(n_embd, n_embd, bias=False)
+        self.receptance = nn.Linear(n_embd, n_embd, bias=False)
+        self.key_norm = nn.LayerNorm(n_embd) if key_norm else None
+        self.output = nn.Linear(n_embd, n_embd, bias=False)
+
+    def forward(self, x, patch_resolution):
+        B, T, C = x.shape
+        if self.shift_pixel > 0:
+            xk, xv, xr = _mix(x, [self.spatial_mix_k, self.spatial_mix_v, self.spatial_mix_r], self.shift_pixel,
+                              self.channel_gamma, patch_resolution, self.fused_shift)
+        else:
+            xk = xv = xr = x
+        k, v = self.key(xk), self.value(xv)
+        sr = torch.sigmoid(self.receptance(xr))
+        y = RUN_CUDA(self.spatial_decay / T, self.spatial_first / T, k, v)      # vrwkv.py:183
+        y = y.to(sr.dtype)
+        if self.key_norm is not None:
+            y = self.key_norm(y)
+        return self.output(sr * y)
+
+
+class VRWKV_ChannelMix(nn.Module):
+    def __init__(self, n_embd, n_layer, layer_id, channel_gamma=1 / 4, shift_pixel=1, hidden_rate=4, key_norm=False,
+                 fused_shift=True):
+        super().__init__()
+        self.shift_pixel, self.channel_gamma, self.fused_shift = shift_pixel, channel_gamma, fused_shift
+        r10 = 1.0 - layer_id / n_layer
+        x = (torch.arange(n_embd, dtype=torch.float32) / n_embd).reshape(1, 1, n_embd)
+        self.spatial_mix_k = nn.Parameter(torch.pow(x, r10))
+        self.spatial_mix_r = nn.Parameter(torch.pow(x, r10))
+        hidden = hidden_rate * n_embd
+        self.key = nn.Linear(n_embd, hidden, bias=False)
+        self.key_norm = nn.LayerNorm(hidden) if key_norm else None
+        self.receptance = nn.Linear(n_embd, n_embd, bias=False)
+        self.value = nn.Linear(hidden, n_embd, bias=False)
+
+    def forward(self, x, patch_resolution):
+        if self.shift_pixel > 0:
+            xk, xr = _mix(x, [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel, self.channel_gamma,
+                          patch_resolution, self.fused_shift)
+        else:
+            xk = xr = x
+        k = torch.square(torch.relu(self.key(xk)))
+        if self.key_norm is not None:
+            k = self.key_norm(k)
+        return torch.sigmoid(self.receptance(xr)) * self.value(k)
+
+
+class Block(nn.Module):
+    def __init__(self, n_embd, n_layer, layer_id, channel_gamma=1 / 4, shift_pixel=1, hidden_rate=4, init_values=None,
+                 post_norm=False, key_norm=False, fused_shift=True):
+        super().__init__()
+        self.layer_id, self.post_norm = layer_id, post_norm
+        self.ln1, self.ln2 = nn.LayerNorm(n_embd), nn.LayerNorm(n_embd)
+        if layer_id == 0:
+            self.ln0 = nn.LayerNorm(n_embd)
+        self.att = VRWKV_SpatialMix(n_embd, n_layer, layer_id, channel_gamma, shift_pixel, key_norm, fused_shift)
+        self.ffn = VRWKV_ChannelMix(n_embd, n_layer, layer_id, channel_gamma, shift_pixel, hidden_rate, key_norm, fused_shift)
+        self.layer_scale = init_values is not None
+        if self.layer_scale:
+            self.gamma1 = nn.Parameter(init_values * torch.ones(n_embd))
+            self.gamma2 = nn.Parameter(init_values * torch.ones(n_embd))
+
+    def forward(self, x, patch_resolution):
+        if self.layer_id == 0:
+            x = self.ln0(x)
+        g1 = self.gamma1 if self.layer_scale else 1.0
+        g2 = self.gamma2 if self.layer_scale else 1.0
+        if self.post_norm:                                   # vrwkv.py:300-306
+            x = x + g1 * self.ln1(self.att(x, patch_resolution))
+            x = x + g2 * self.ln2(self.ffn(x, patch_resolution))
+        else:
+            x = x + g1 * self.att(self.ln1(x), patch_resolution)
+            x = x + g2 * self.ffn(self.ln2(x), patch_resolution)
+        return x
+
+
+class VRWKV(nn.Module):
+    """vrwkv.py:322-432 without the mmcv base classes; returns the last feature map (B, C, Hp, Wp)."""
+
+    def __init__(self, img_size=224, patch_size=16, in_channels=3, embed_dims=256, depth=12, channel_gamma=1 / 4,
+                 shift_pixel=1, post_norm=False, key_norm=False, init_values=None, hidden_rate=4, final_norm=True,
+                 interpolate_mode="bicubic", fused_shift=True):
+        super().__init__()
+        self.patch_size = patch_size
+        self.patch_embed = nn.Conv2d(in_channels, embed_dims, kernel_size=patch_size, stride=patch_size, bias=True)
+        self.patch_resolution = (img_size // patch_size, img_size // patch_size)
+        self.pos_embed = nn.Parameter(torch.zeros(1, self.patch_resolution[0] * self.patch_resolution[1], embed_dims))
+        self.interpolate_mode = interpolate_mode
+        self.layers = nn.ModuleList([
+            Block(embed_dims, depth, i, channel_gamma, shift_pixel, hidden_rate, init_values, post_norm, key_norm,
+                  fused_shift) for i in range(depth)])
+        self.final_norm = final_norm
+        if final_norm:
+            self.ln1 = nn.LayerNorm(embed_dims)
+
+    def forward(self, img):
+        x = self.patch_embed(img)
+        res = (x.shape[2], x.shape[3])
+        x = x.flatten(2).transpose(1, 2)
+        x = x + resize_pos_embed(self.pos_embed, self.patch_resolution, res, self.interpolate_mode).to(x.dtype)
+        for layer in self.layers:
+            x = layer(x, res)
+        if self.final_norm:
+            x = self.ln1(x)
+        B, _, C = x.shape
+        return x.reshape(B, res[0], res[1], C).permute(0, 3, 1, 2)
+
+
+def vrwkv_l(**kw):
+    """VRWKV-L as fine-tuned at 384x384: classification_internimage/configs/vrwkv_l_22kto1k_384.yaml:10-28
+    (pre-training grid 192/16 = 12x12, interpolated to 24x24; K_NORM defaults to True, config.py:82)."""
+    cfg = dict(img_size=192, patch_size=16, embed_dims=1024, depth=24, post_norm=True, init_values=1e-5,
+               hidden_rate=4, key_norm=True, final_norm=True)
+    cfg.update(kw)
+    return VRWKV(**cfg)

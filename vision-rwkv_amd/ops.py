@@ -8,6 +8,8 @@ Mirrors
 with the same argument meaning, output dtype rule and error behaviour (RuntimeError for
 non-device / non-contiguous tensors).
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -237,3 +239,42 @@ class WKV_6(torch.autograd.Function):
 def RUN_CUDA_RWKV6(B, T, C, H, r, k, v, w, u):
     """vrwkv6.py:72-73."""
     return WKV_6.apply(B, T, C, H, r, k, v, w, u)
+
+
+def q_shift(input, shift_pixel=1, gamma=1 / 4, patch_resolution=None):
+    """q_shift of vrwkv.py:68-79 in plain tensor ops (used where gradients are needed)."""
+    assert gamma <= 1 / 4
+    B, N, C = input.shape
+    x = input.transpose(1, 2).reshape(B, C, patch_resolution[0], patch_resolution[1])
+    H, W = patch_resolution
+    g = int(C * gamma)
+    out = torch.zeros_like(x)
+    out[:, 0:g, :, shift_pixel:W] = x[:, 0:g, :, 0:W - shift_pixel]
+    out[:, g:2 * g, :, 0:W - shift_pixel] = x[:, g:2 * g, :, shift_pixel:W]
+    out[:, 2 * g:3 * g, shift_pixel:H, :] = x[:, 2 * g:3 * g, 0:H - shift_pixel, :]
+    out[:, 3 * g:4 * g, 0:H - shift_pixel, :] = x[:, 3 * g:4 * g, shift_pixel:H, :]
+    out[:, 4 * g:, ...] = x[:, 4 * g:, ...]
+    return out.flatten(2).transpose(1, 2)
+
+
+def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, head_dim=0):
+    """One HIP kernel for q_shift + the token-mix lerps: returns [x*m + q_shift(x)*(1-m) for m in mixes]
+    (vrwkv.py:160-163 / :248-250).  mixes: 1..3 tensors of C elements.  head_dim=64 gives the per-head
+    q_shift_multihead of vrwkv6.py:75-100 (a trailing class token is passed through).  Forward only."""
+    _check_input(x, "x")
+    if x.dim() != 3 or x.dtype not in _DT:
+        raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
+    B, T, C = x.shape
+    Hp, Wp = patch_resolution
+    mix = torch.stack([m.reshape(-1).float() for m in mixes]).contiguous().to(x.device)
+    if mix.shape[1] != C:
+        raise RuntimeError("every mix vector must have C elements")
+    outs = [torch.empty_like(x) for _ in mixes]
+    if x.numel() == 0:
+        return outs
+    ptrs = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+    g = head_dim // 4 if head_dim else int(C * gamma)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().vrwkv_qshift_mix(x.data_ptr(), mix.data_ptr(), ptrs, len(outs), B, T, C, Hp, Wp,
+                                               shift_pixel, g, head_dim, _DT[x.dtype], _stream_ptr(x.device)))
+    return outs
