@@ -101,6 +101,45 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
     return out
 
 
+def backbone_section(torch, ops, steps, warmup):
+    """VRWKV-L forward (24 blocks, C=1024, 384x384 input -> T=576) at batch 32 in bf16, random weights:
+    ms per forward, and the share of it spent in the 24 Bi-WKV calls (timed alone at the same shape)."""
+    dev = torch.device("cuda:0")
+    Bn, S = 32, 384
+    torch.manual_seed(0)
+    net = ops.vrwkv_l().to(dev).eval().bfloat16()
+    img = torch.randn(Bn, 3, S, S, device=dev, dtype=torch.bfloat16)
+
+    def timed(fn, n, wu):
+        for _ in range(wu):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    with torch.no_grad():
+        ms_fwd = timed(lambda: net(img), steps, warmup)
+        for m in net.modules():
+            if hasattr(m, "fused_shift"):
+                m.fused_shift = False
+        ms_fwd_eager_shift = timed(lambda: net(img), steps, warmup)
+        Tn, Cn = (S // 16) ** 2, 1024
+        att = net.layers[0].att
+        k = torch.randn(Bn, Tn, Cn, device=dev, dtype=torch.bfloat16)
+        v = torch.randn(Bn, Tn, Cn, device=dev, dtype=torch.bfloat16)
+        w, u = (att.spatial_decay / Tn).float(), (att.spatial_first / Tn).float()
+        ms_wkv = timed(lambda: ops.bi_wkv_forward(w, u, k, v), 24 * steps, 24 * warmup) * 24
+    return {"workload": f"VRWKV-L forward, batch {Bn}, {S}x{S}, T={Tn}, C={Cn}, 24 blocks, bf16, random weights",
+            "ms_per_forward": round(ms_fwd, 3), "images_per_s": round(Bn / ms_fwd * 1e3, 1),
+            "ms_per_forward_unfused_shift": round(ms_fwd_eager_shift, 3),
+            "biwkv_ms_per_forward": round(ms_wkv, 3), "biwkv_share": round(ms_wkv / ms_fwd, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +148,7 @@ def main():
     ap.add_argument("--io", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-wkv6", action="store_true", help="skip the secondary wkv6 measurement")
+    ap.add_argument("--no-backbone", action="store_true", help="skip the VRWKV-L whole-forward measurement")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -210,6 +250,8 @@ def main():
         out["cpu_baseline"] = cb
     if not args.no_wkv6:
         out["wkv6"] = wkv6_section(torch, ops, max(args.steps, 10), max(args.warmup // 5, 3), not args.no_cpu_baseline)
+    if not args.no_backbone:
+        out["backbone"] = backbone_section(torch, ops, 5, 3)
     print(json.dumps(out))
 
 
