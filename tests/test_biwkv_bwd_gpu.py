@@ -86,3 +86,54 @@ def test_autograd_function_end_to_end(ops):
     ref = biwkv.biwkv_grads_closed(w.numpy(), u.numpy(), k.numpy(), v.numpy(), gy.numpy())
     for leaf, r in zip(leaves, ref):
         assert rel_err(leaf.grad.cpu().numpy(), r) <= 2e-4
+
+
+def test_tiled_kernel_equals_sequential_kernel_full_size(ops, monkeypatch):
+    """VRWKV-B shape: the tiled kernel against the sequential one (forced through the environment), and
+    the sum identities that hold at any size."""
+    B, T, C = 64, 196, 768
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(B, T, C, generator=g).cuda()
+    v = torch.randn(B, T, C, generator=g).cuda()
+    gy = torch.randn(B, T, C, generator=g).cuda()
+    w = ((torch.rand(C, generator=g) * 8 - 5) / T).cuda()
+    u = (torch.rand(C, generator=g) - 0.5).cuda()
+    got = ops.bi_wkv_backward(w, u, k, v, gy)
+    monkeypatch.setenv("VRWKV_BIWKV_BWD_PATH", "serial")
+    ref = ops.bi_wkv_backward(w, u, k, v, gy)
+    torch.cuda.synchronize()
+    # two fp32 evaluations (the sequential one renormalises at every token and is the less accurate)
+    for a, b, name in zip(got, ref, ("gw", "gu", "gk", "gv")):
+        assert rel_err(a.cpu().numpy(), b.cpu().numpy()) <= 5e-4, name
+    # float64 closed form on a slice (gk, gv of a sequence depend on that sequence only)
+    from oracle import biwkv
+    sl = (slice(0, 2), slice(None), slice(640, 704))
+    f = lambda x: x.cpu().numpy()
+    _, _, rk, rv = biwkv.biwkv_grads_closed(f(w[640:704]), f(u[640:704]), f(k[sl]), f(v[sl]), f(gy[sl]))
+    assert rel_err(f(got[2][sl]), rk) <= 1e-4 and rel_err(f(got[3][sl]), rv) <= 1e-4
+    gk, gv = got[2], got[3]
+    assert (gv.sum(1) - gy.sum(1)).abs().max().item() <= 1e-4 * gy.abs().sum(1).max().item()
+    assert gk.sum(1).abs().max().item() <= 1e-4 * gk.abs().max().item() * T ** 0.5
+
+
+@pytest.mark.parametrize("T", [29, 100, 224, 225, 300])
+def test_wave_scales_far_apart_and_sequence_lengths(ops, T):
+    """k jumps by +-60 between token ranges (every wave gets its own reference exponent, rescaled exactly
+    when aggregates cross waves); T = 224 is the longest tiled case, 225 and 300 take the sequential kernel."""
+    from oracle import biwkv
+    B, C = 2, 64
+    rng = np.random.default_rng(T)
+    k = rng.standard_normal((B, T, C)).astype(np.float32)
+    k[:, T // 3: T // 2] += 60.0
+    k[:, T // 2: (2 * T) // 3] -= 60.0
+    k[1, 5] += 80.0
+    v, gy = (rng.standard_normal((B, T, C)).astype(np.float32) for _ in range(2))
+    w = (rng.uniform(-5, 3, C) / T).astype(np.float32)
+    u = rng.uniform(-1, 1, C).astype(np.float32)
+    gw, gu, gk, gv, *_ = run(ops, w, u, k, v, gy)
+    rw, ru, rk, rv = biwkv.biwkv_grads_closed(w, u, k, v, gy)
+    assert np.isfinite(gk).all() and np.isfinite(gv).all()
+    # where one token outweighs all others, y_t ~ v_i for every t and gk_i = sum_t z_t W[t,i] (v_i - y_t)
+    # cancels to ~1e-6 of its terms: fp32 keeps 5e-4 of the tensor's rms there (both kernels), not 1e-4
+    assert rel_err(gk, rk) <= 5e-4 and rel_err(gv, rv) <= 5e-4
+    assert rel_err(gw, rw) <= 5e-4 and rel_err(gu, ru) <= 5e-4

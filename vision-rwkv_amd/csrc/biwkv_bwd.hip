@@ -18,106 +18,24 @@
 // gw and gu are reduced over the batch by a second small kernel (deterministic, no atomics).
 // The reference needs 3 scratch tensors and atomicAdd (bi_wkv_kernel.cu:303-304, 415-417);
 // here the workspace is 5 floats per element + 2*B*C.
-#include "vrwkv_common.h"
+#include "biwkv_bwd_serial.h"
+#include "biwkv_bwd_tile.h"
 
 namespace vrwkv {
 namespace {
 
-// (mantissas..., exponent) <- decay by one token, then add a term with exponent e
-struct Scan {
-    float s0 = 0.f, s1 = 0.f, l0 = 0.f, l1 = 0.f, p = NEG_BIG;   // sums of z, z*y; distance-weighted sums
-    __device__ __forceinline__ void push(float om, float z, float zy, float e) {
-        const float pw = fmaxf(p - om, NEG_BIG);
-        const float q = fmaxf(pw, e);
-        const float c1 = fast_exp2(pw - q), c2 = fast_exp2(e - q);
-        l0 = c1 * (l0 + s0);                 // distances grow by one; the new term enters at distance 0
-        l1 = c1 * (l1 + s1);
-        s0 = c1 * s0 + c2 * z;
-        s1 = c1 * s1 + c2 * zy;
-        p = q;
-    }
-};
+using namespace biwkv_bwd_detail;
 
 template <typename IO>
 __global__ __launch_bounds__(64)
-void biwkv_bwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
-                      const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
-                      IO* __restrict__ gk_, IO* __restrict__ gv_, float* __restrict__ ws,
-                      float* __restrict__ gw_part, float* __restrict__ gu_part, int B, int T, int C)
+void biwkv_bwd_serial_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
+                             const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
+                             IO* __restrict__ gk_, IO* __restrict__ gv_, float* __restrict__ ws,
+                             float* __restrict__ gw_part, float* __restrict__ gu_part, int B, int T, int C)
 {
     const int c = blockIdx.x * 64 + threadIdx.x;
-    const int b = blockIdx.y;
     if (c >= C) return;
-    const float om = w_[c] * LOG2E, mu = u_[c] * LOG2E;
-    const size_t base = (size_t)b * T * C + c;
-    const size_t plane = (size_t)B * T * C;
-    float* W0 = ws;                 // a      -> later z mantissa
-    float* W1 = ws + plane;         // b      -> later y
-    float* W2 = ws + 2 * plane;     // p      -> later m (exponent of z)
-    float* W3 = ws + 3 * plane;     // partial gv
-    float* W4 = ws + 4 * plane;     // partial gk
-
-    // ---- pass A: past state before each token ----
-    {
-        float a = 0.f, bb = 0.f, p = NEG_BIG;
-        for (int t = 0; t < T; ++t) {
-            const size_t o = base + (size_t)t * C;
-            W0[o] = a; W1[o] = bb; W2[o] = p;
-            const float kap = to_f32(k_[o]) * LOG2E, v = to_f32(v_[o]);
-            const float pw = fmaxf(p - om, NEG_BIG), q = fmaxf(pw, kap);
-            const float e1 = fast_exp2(pw - q), e2 = fast_exp2(kap - q);
-            a = e1 * a + e2 * v; bb = e1 * bb + e2; p = q;
-        }
-    }
-    float gu_acc = 0.f, gw_acc = 0.f;
-    // ---- pass B: future state, y, z; future scans ----
-    {
-        float cc = 0.f, d = 0.f, o_ = NEG_BIG;
-        Scan f;
-        for (int t = T - 1; t >= 0; --t) {
-            const size_t o = base + (size_t)t * C;
-            const float kap = to_f32(k_[o]) * LOG2E, v = to_f32(v_[o]), gy = to_f32(gy_[o]);
-            const float a = W0[o], bb = W1[o], p = W2[o];
-            const float uk = mu + kap;
-            const float m = fmaxf(fmaxf(p, o_), uk);
-            const float ea = fast_exp2(p - m), ec = fast_exp2(o_ - m), eu = fast_exp2(uk - m);
-            const float den = ea * bb + ec * d + eu;
-            const float y = (ea * a + ec * cc + eu * v) / den;
-            const float z = gy / den;                       // z_t = z * 2^-m in absolute scale
-            const float zy = z * y;
-            // contributions of later tokens (t' > t) and of the token itself
-            const float sf = fast_exp2(kap + f.p);          // 2^(kappa_i + exponent of the scan)
-            const float self = z * eu;
-            const float gv = sf * f.s0 + self;
-            const float gk = v * gv - (sf * f.s1 + self * y);
-            gu_acc += self * (v - y);
-            gw_acc -= sf * (v * f.l0 - f.l1);
-            W3[o] = gv; W4[o] = gk;
-            W0[o] = z; W1[o] = y; W2[o] = m;
-            // this token joins the future of the earlier ones
-            f.push(om, z, zy, -m);
-            const float pw = fmaxf(o_ - om, NEG_BIG), q = fmaxf(pw, kap);
-            const float e1 = fast_exp2(pw - q), e2 = fast_exp2(kap - q);
-            cc = e1 * cc + e2 * v; d = e1 * d + e2; o_ = q;
-        }
-    }
-    // ---- pass C: past scans, final gk, gv ----
-    {
-        Scan g;
-        for (int t = 0; t < T; ++t) {
-            const size_t o = base + (size_t)t * C;
-            const float kap = to_f32(k_[o]) * LOG2E, v = to_f32(v_[o]);
-            const float z = W0[o], y = W1[o], m = W2[o];
-            const float sp = fast_exp2(kap + g.p);
-            const float gvp = sp * g.s0;
-            gv_[o] = from_f32<IO>(W3[o] + gvp);
-            gk_[o] = from_f32<IO>(W4[o] + v * gvp - sp * g.s1);
-            gw_acc -= sp * (v * g.l0 - g.l1);
-            g.push(om, z, z * y, -m);
-        }
-    }
-    gw_part[(size_t)b * C + c] = gw_acc;
-    gu_part[(size_t)b * C + c] = gu_acc;
+    biwkv_bwd_serial_seq<IO>(w_, u_, k_, v_, gy_, gk_, gv_, ws, gw_part, gu_part, B, T, C, blockIdx.y, c);
 }
 
 __global__ void biwkv_bwd_reduce_kernel(const float* __restrict__ gw_part, const float* __restrict__ gu_part,
@@ -152,9 +70,33 @@ int launch(const float* w, const float* u, const void* k, const void* v, const v
     const size_t plane = (size_t)B * T * C;
     float* gw_part = ws + 5 * plane;
     float* gu_part = gw_part + (size_t)B * C;
-    hipLaunchKernelGGL((biwkv_bwd_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
-                       static_cast<const IO*>(k), static_cast<const IO*>(v), static_cast<const IO*>(gy),
-                       static_cast<IO*>(gk), static_cast<IO*>(gv), ws, gw_part, gu_part, B, T, C);
+    const IO* kk = static_cast<const IO*>(k);
+    const IO* vv = static_cast<const IO*>(v);
+    const IO* gg = static_cast<const IO*>(gy);
+    IO* ok = static_cast<IO*>(gk);
+    IO* ov = static_cast<IO*>(gv);
+    // sequences that fit one workgroup (8 waves x L tokens) take the tiled kernel
+    static const int kL[] = {4, 8, 16, 28};
+    int L = 0;
+    const char* path = getenv("VRWKV_BIWKV_BWD_PATH");       // "serial" forces the sequential kernel (testing)
+    if (!(path && path[0] == 's'))
+        for (int i = 3; i >= 0; --i)
+            if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX) L = kL[i];   // smallest L that fits: most waves per tile
+    if (L) {
+        const int S = (T + L - 1) / L;
+        const int n_ctile = (C + WAVE - 1) / WAVE;
+        const int n_tiles = B * n_ctile;
+        const int per_cu = BWD_SMAX / S > 0 ? BWD_SMAX / S : 1;
+        int grid = biwkv_fwd_detail::num_cus() * per_cu;
+        if (grid > n_tiles) grid = n_tiles;
+#define VRWKV_BWD_CASE(LL) case LL: hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, LL>), dim3(grid), dim3(S * WAVE), 0, st, \
+                           w, u, kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C, n_ctile, n_tiles); break;
+        switch (L) { VRWKV_BWD_CASE(4) VRWKV_BWD_CASE(8) VRWKV_BWD_CASE(16) VRWKV_BWD_CASE(28) }
+#undef VRWKV_BWD_CASE
+    } else {
+        hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
+                           kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C);
+    }
     hipLaunchKernelGGL(biwkv_bwd_reduce_kernel, dim3((C + 255) / 256), dim3(256), 0, st, gw_part, gu_part, gw, gu, B, C);
     return check_launch("biwkv_bwd");
 }

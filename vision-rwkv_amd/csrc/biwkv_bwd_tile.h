@@ -1,0 +1,284 @@
+// Bi-WKV backward, tiled kernel for sequences that fit one workgroup (T <= 8 waves x 28 tokens).
+//
+// Same decomposition as the forward kernel: lane = channel, wave = L consecutive tokens in registers,
+// workgroup = one (batch, 64 channels) tile, persistent workgroups walking the tiles.  k, v, gy are
+// read from HBM once and gk, gv written once; nothing else touches HBM except 2 floats per (b, c).
+//
+// With E_i = e^{k_i}, g = e^{-w}, cu = e^{u}:
+//   phase 1 (the forward):  D_t = sum_{i<t} g^{t-i-1} E_i + sum_{i>t} g^{i-t-1} E_i + cu E_t, N_t likewise
+//                           with E_i v_i;  y_t = N_t / D_t,  z_t = gy_t / D_t
+//   phase 2 (its adjoint):  Z_i = sum_{t<i} g^{i-t-1} z_t + sum_{t>i} g^{t-i-1} z_t + cu z_i, ZY_i likewise
+//                           with z_t y_t;  gv_i = E_i Z_i,  gk_i = v_i gv_i - E_i ZY_i
+//   gu = sum_i cu E_i (v_i z_i - z_i y_i)
+//   gw = - sum_i E_i (v_i Lz_i - Lzy_i),  Lz_i = sum_{t!=i} (|t-i|-1) g^{|t-i|-1} z_t  (running sums
+//        l <- g (l + s) next to s <- g s + z, so no per-token storage)
+// Each phase is: per-wave chunk aggregates -> one LDS exchange -> carry-in from the other waves ->
+// ascending sweep (past side) -> descending sweep (future side).
+//
+// Scaling: as in the forward's plain-sum path every wave works in units of 2^Rw, Rw = ceil(max kappa)
+// over its tokens, and z carries 2^-Re with Re = max(Rw, R - 100) the scale its denominators were
+// actually formed at.  Another wave's z-aggregates are brought over with the exact factor
+// 2^(Rw_mine - Re_theirs): that is the same power of two by which my E entered their denominators, so
+// the product stays below |gy| 2^41 and nothing overflows.  Tiles outside the plain-sum regime
+// (|omega| (T+1) + |mu| > 40) are left to the sequential kernel, which renormalises at every token.
+#pragma once
+#include "biwkv_fwd_impl.h"
+#include "biwkv_bwd_serial.h"
+
+namespace vrwkv {
+namespace biwkv_bwd_detail {
+
+using namespace biwkv_fwd_detail;
+
+constexpr int BWD_SMAX = 8;
+
+template <typename IO>
+__device__ __forceinline__ float unpack1(typename BufRaw<sizeof(IO)>::type raw) {
+    IO tmp;
+    __builtin_memcpy(&tmp, &raw, sizeof(raw));
+    return to_f32(tmp);
+}
+template <typename IO>
+__device__ __forceinline__ void store1(__amdgpu_buffer_rsrc_t r, unsigned voff, float x) {
+    const IO tmp = from_f32<IO>(x);
+    typename BufRaw<sizeof(IO)>::type raw;
+    __builtin_memcpy(&raw, &tmp, sizeof(raw));
+    BufRaw<sizeof(IO)>::template st<CPOL_NT>(raw, r, voff, 0);
+}
+
+// True when this wave's 64 channels may use the plain-sum path (wave-uniform).
+__device__ __forceinline__ bool bwd_tile_is_fast(float om, float mu, int T) {
+    const bool bad = !(fabsf(om) * (float)(T + 1) + fabsf(mu) <= FAST_LIMIT);
+    return __builtin_amdgcn_ballot_w64(bad) == 0ull;
+}
+
+struct ZScan {
+    float s0 = 0.f, s1 = 0.f, l0 = 0.f, l1 = 0.f;
+    __device__ __forceinline__ void push(float g, float z, float zy) {
+        l0 = g * (l0 + s0);
+        l1 = g * (l1 + s1);
+        s0 = fmaf(g, s0, z);
+        s1 = fmaf(g, s1, zy);
+    }
+    // n tokens of another wave pass in between: decay, then add that wave's own sums
+    __device__ __forceinline__ void hop(float G, float n, float a0, float a1, float b0, float b1) {
+        l0 = fmaf(G, fmaf(n, s0, l0), b0);
+        l1 = fmaf(G, fmaf(n, s1, l1), b1);
+        s0 = fmaf(G, s0, a0);
+        s1 = fmaf(G, s1, a1);
+    }
+};
+
+template <typename IO, int L>
+__global__ __launch_bounds__(BWD_SMAX * WAVE)
+void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
+                           const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
+                           IO* __restrict__ gk_, IO* __restrict__ gv_,
+                           float* __restrict__ ws, float* __restrict__ gw_part, float* __restrict__ gu_part,
+                           int B, int T, int C, int n_ctile, int n_tiles)
+{
+    using Raw = typename BufRaw<sizeof(IO)>::type;
+    __shared__ float s1[BWD_SMAX][5][WAVE];
+    __shared__ float s2[BWD_SMAX][9][WAVE];
+    __shared__ float s3[BWD_SMAX][2][WAVE];
+
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int S = blockDim.x >> 6;
+    const float NEG_INF = -__builtin_inff();
+    const unsigned row = (unsigned)(C * sizeof(IO));
+    const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
+    auto shift_of = [](float d) -> int { return (int)fminf(fmaxf(d, -300.f), 300.f); };
+
+    for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int ctile = tile % n_ctile, b = tile / n_ctile;
+        const int c0 = ctile * WAVE + lane;
+        const bool cok = c0 < C;
+        const int tw = wave * L;
+        const unsigned voff0 = cok ? (unsigned)(((size_t)tw * C + c0) * sizeof(IO)) : OOB_OFFSET;
+        const size_t slab = (size_t)b * T * C;
+        const float om = (cok ? w_[c0] : 0.f) * LOG2E;
+        const float mu = (cok ? u_[c0] : 0.f) * LOG2E;
+        if (!bwd_tile_is_fast(om, mu, T)) continue;          // workgroup-uniform: same channels in every wave
+
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes);
+        const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
+        const __amdgpu_buffer_rsrc_t rg = make_rsrc(gy_ + slab, bytes);
+        Raw Kr[L], Vr[L], Gr[L];
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            const unsigned vo = voff0 + (unsigned)j * row;
+            Kr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rk, vo, 0);
+            Vr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rv, vo, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < L; ++j)
+            Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
+
+        const float gd = fast_exp2(-om), cu = fast_exp2(mu);
+        const float G = fast_exp2(-om * (float)L);
+
+        // ------------------------------ phase 1: the forward ------------------------------
+        float E[L], V[L];
+        float m = NEG_INF;
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            const float kk = unpack1<IO>(Kr[j]);
+            E[j] = (tw + j < T) ? kk : NEG_INF;               // tokens past T: k = -inf
+            V[j] = unpack1<IO>(Vr[j]);
+            m = fmaxf(m, E[j]);
+        }
+        const bool any = m > NEG_INF;
+        const float Rw = any ? ceilf(m * LOG2E) : 0.f;
+        float A = 0.f, Bd = 0.f, Cg = 0.f, Dg = 0.f;
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            E[j] = fast_exp2(fmaf(E[j], LOG2E, -Rw));
+            A = fmaf(gd, A, E[j] * V[j]);
+            Bd = fmaf(gd, Bd, E[j]);
+        }
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j) {
+            Cg = fmaf(gd, Cg, E[j] * V[j]);
+            Dg = fmaf(gd, Dg, E[j]);
+        }
+        s1[wave][0][lane] = A;
+        s1[wave][1][lane] = Bd;
+        s1[wave][2][lane] = any ? Rw : NEG_BIG;
+        s1[wave][3][lane] = Cg;
+        s1[wave][4][lane] = Dg;
+        lds_barrier();
+
+        float a = 0.f, bb = 0.f, c = 0.f, d = 0.f, Re;
+        {
+            float la[BWD_SMAX], lb[BWD_SMAX], lc[BWD_SMAX], ld[BWD_SMAX], lr[BWD_SMAX];
+#pragma unroll
+            for (int s = 0; s < BWD_SMAX; ++s) {
+                const int ss = s < S ? s : S - 1;
+                la[s] = s1[ss][0][lane]; lb[s] = s1[ss][1][lane]; lr[s] = s1[ss][2][lane];
+                lc[s] = s1[ss][3][lane]; ld[s] = s1[ss][4][lane];
+            }
+            float r = NEG_BIG;
+#pragma unroll
+            for (int s = 0; s < BWD_SMAX; ++s) r = fmaxf(r, lr[s]);
+            r = (r > NEG_BIG) ? r : 0.f;
+#pragma unroll
+            for (int s = 0; s < BWD_SMAX; ++s)
+                if (s < wave) {
+                    const int sh = shift_of(lr[s] - r);
+                    a = fmaf(G, a, ldexpf(la[s], sh));
+                    bb = fmaf(G, bb, ldexpf(lb[s], sh));
+                }
+#pragma unroll
+            for (int s = BWD_SMAX - 1; s >= 0; --s)
+                if (s > wave && s < S) {
+                    const int sh = shift_of(lr[s] - r);
+                    c = fmaf(G, c, ldexpf(lc[s], sh));
+                    d = fmaf(G, d, ldexpf(ld[s], sh));
+                }
+            const float upf = fminf(r - Rw, 100.f);
+            const int up = (int)upf;
+            a = ldexpf(a, up); bb = ldexpf(bb, up); c = ldexpf(c, up); d = ldexpf(d, up);
+            Re = r - upf;                                     // the scale the carried terms really have
+        }
+
+        float Z[L], ZY[L];                                    // first N, D partials, then z and z*y
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            const float ev = E[j] * V[j];
+            Z[j] = fmaf(cu, ev, a);
+            ZY[j] = fmaf(cu, E[j], bb);
+            a = fmaf(gd, a, ev);
+            bb = fmaf(gd, bb, E[j]);
+        }
+        float gu_acc = 0.f, gw_acc = 0.f;
+        ZScan fl;                                             // local future-side sums, zero carry
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j) {
+            const float ev = E[j] * V[j];
+            const float rD = (tw + j < T) ? fast_rcp(ZY[j] + d) : 0.f;   // tokens past T contribute nothing
+            const float y = (Z[j] + c) * rD;
+            const float z = unpack1<IO>(Gr[j]) * rD;
+            const float zy = z * y;
+            c = fmaf(gd, c, ev);
+            d = fmaf(gd, d, E[j]);
+            Z[j] = z;
+            ZY[j] = zy;
+            gu_acc = fmaf(cu * E[j], fmaf(V[j], z, -zy), gu_acc);
+            fl.push(gd, z, zy);
+        }
+        ZScan pl;                                             // local past-side sums
+#pragma unroll
+        for (int j = 0; j < L; ++j) pl.push(gd, Z[j], ZY[j]);
+
+        // ------------------------------ phase 2: the adjoint ------------------------------
+        s2[wave][0][lane] = pl.s0; s2[wave][1][lane] = pl.s1; s2[wave][2][lane] = pl.l0; s2[wave][3][lane] = pl.l1;
+        s2[wave][4][lane] = fl.s0; s2[wave][5][lane] = fl.s1; s2[wave][6][lane] = fl.l0; s2[wave][7][lane] = fl.l1;
+        s2[wave][8][lane] = Re;
+        lds_barrier();
+
+        ZScan p, f;
+        {
+            const float nL = (float)L;
+#pragma unroll
+            for (int s = 0; s < BWD_SMAX; ++s)
+                if (s < wave) {
+                    const int sh = shift_of(Rw - s2[s][8][lane]);
+                    p.hop(G, nL, ldexpf(s2[s][0][lane], sh), ldexpf(s2[s][1][lane], sh),
+                          ldexpf(s2[s][2][lane], sh), ldexpf(s2[s][3][lane], sh));
+                }
+#pragma unroll
+            for (int s = BWD_SMAX - 1; s >= 0; --s)
+                if (s > wave && s < S) {
+                    const int sh = shift_of(Rw - s2[s][8][lane]);
+                    f.hop(G, nL, ldexpf(s2[s][4][lane], sh), ldexpf(s2[s][5][lane], sh),
+                          ldexpf(s2[s][6][lane], sh), ldexpf(s2[s][7][lane], sh));
+                }
+        }
+        float GV[L], GK[L];
+#pragma unroll
+        for (int j = 0; j < L; ++j) {
+            GV[j] = fmaf(cu, Z[j], p.s0);
+            GK[j] = fmaf(cu, ZY[j], p.s1);
+            gw_acc = fmaf(-E[j], fmaf(V[j], p.l0, -p.l1), gw_acc);
+            p.push(gd, Z[j], ZY[j]);
+        }
+        const __amdgpu_buffer_rsrc_t rgk = make_rsrc(gk_ + slab, bytes);
+        const __amdgpu_buffer_rsrc_t rgv = make_rsrc(gv_ + slab, bytes);
+#pragma unroll
+        for (int j = L - 1; j >= 0; --j) {
+            const float gv = E[j] * (GV[j] + f.s0);
+            const float gk = fmaf(V[j], gv, -E[j] * (GK[j] + f.s1));
+            gw_acc = fmaf(-E[j], fmaf(V[j], f.l0, -f.l1), gw_acc);
+            f.push(gd, Z[j], ZY[j]);
+            const unsigned vo = voff0 + (unsigned)j * row;    // tokens >= T fall outside the descriptor
+            store1<IO>(rgv, vo, gv);
+            store1<IO>(rgk, vo, gk);
+        }
+
+        // per-(b, c) partial sums of gw, gu: over this wave's tokens, then over the waves
+        s3[wave][0][lane] = gw_acc;
+        s3[wave][1][lane] = gu_acc;
+        lds_barrier();
+        if (wave == 0 && cok) {
+            float sw = 0.f, su = 0.f;
+            for (int s = 0; s < S; ++s) { sw += s3[s][0][lane]; su += s3[s][1][lane]; }
+            gw_part[(size_t)b * C + c0] = sw;
+            gu_part[(size_t)b * C + c0] = su;
+        }
+    }
+
+    // second walk: tiles outside the plain-sum regime, one wave per tile, sequential form
+    for (int tile = blockIdx.x * S + wave; tile < n_tiles; tile += gridDim.x * S) {
+        const int ctile = tile % n_ctile, b = tile / n_ctile;
+        const int c0 = ctile * WAVE + lane;
+        const bool cok = c0 < C;
+        const float om = (cok ? w_[c0] : 0.f) * LOG2E;
+        const float mu = (cok ? u_[c0] : 0.f) * LOG2E;
+        if (bwd_tile_is_fast(om, mu, T)) continue;
+        if (cok) biwkv_bwd_serial_seq<IO>(w_, u_, k_, v_, gy_, gk_, gv_, ws, gw_part, gu_part, B, T, C, b, c0);
+    }
+}
+
+}  // namespace biwkv_bwd_detail
+}  // namespace vrwkv
