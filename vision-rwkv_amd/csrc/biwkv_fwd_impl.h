@@ -44,8 +44,6 @@ namespace biwkv_fwd_detail {
 
 constexpr float FAST_LIMIT = 40.0f;
 constexpr int NSLOT = 6;   // workspace floats per (b, super-chunk, channel): A, B, pA|R, Cg, D, pC
-constexpr unsigned OOB_OFFSET = 0x80000000u;   // byte offset no descriptor here reaches
-constexpr unsigned CPOL_NT = 2;                // gfx94x/gfx950 cache policy bit: non-temporal (data streamed once)
 
 // Waves per workgroup: at most 8, i.e. two per SIMD, which leaves every wave 256 VGPRs -- enough
 // for the longest chunk (28 tokens: k, v, two partial arrays and the prefetched k, v of the next
@@ -76,29 +74,6 @@ __device__ __forceinline__ void tri_merge(float& a, float& b, float& p, float om
     p = q;
 }
 
-// ---- raw buffer access: VEC elements of IO at byte offset voff (+ scalar soff) ----------
-template <int BYTES> struct BufRaw;
-template <> struct BufRaw<2> {
-    using type = unsigned short;
-    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b16(r, v, s, CP); }
-    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b16(d, r, v, s, CP); }
-};
-template <> struct BufRaw<4> {
-    using type = unsigned int;
-    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b32(r, v, s, CP); }
-    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b32(d, r, v, s, CP); }
-};
-template <> struct BufRaw<8> {
-    typedef unsigned int type __attribute__((ext_vector_type(2)));
-    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b64(r, v, s, CP); }
-    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b64(d, r, v, s, CP); }
-};
-template <> struct BufRaw<16> {
-    typedef unsigned int type __attribute__((ext_vector_type(4)));
-    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b128(r, v, s, CP); }
-    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b128(d, r, v, s, CP); }
-};
-
 // Raw (still packed) registers of one token: converted to fp32 only when consumed, so a
 // prefetched 16-bit tile costs half the registers.
 template <typename IO, int VEC> struct Packed { typename BufRaw<sizeof(IO) * VEC>::type raw; };
@@ -118,10 +93,6 @@ __device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, unsigned vof
     typename BufRaw<sizeof(IO) * VEC>::type raw;
     __builtin_memcpy(&raw, tmp, sizeof(raw));
     BufRaw<sizeof(IO) * VEC>::template st<CPOL_NT>(raw, r, voff, 0);
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
 struct TileGeom {

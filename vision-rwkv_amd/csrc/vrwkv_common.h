@@ -60,6 +60,36 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
+
+// ---- raw buffer access (descriptor + 32-bit byte offsets; out-of-range accesses are dropped by the
+//      hardware: loads return 0, stores do nothing) -------------------------------------------------
+constexpr unsigned OOB_OFFSET = 0x80000000u;   // byte offset no descriptor here reaches
+constexpr unsigned CPOL_NT = 2;                // gfx94x/gfx950 cache policy bit: non-temporal (data streamed once)
+template <int BYTES> struct BufRaw;
+template <> struct BufRaw<2> {
+    using type = unsigned short;
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b16(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b16(d, r, v, s, CP); }
+};
+template <> struct BufRaw<4> {
+    using type = unsigned int;
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b32(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b32(d, r, v, s, CP); }
+};
+template <> struct BufRaw<8> {
+    typedef unsigned int type __attribute__((ext_vector_type(2)));
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b64(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b64(d, r, v, s, CP); }
+};
+template <> struct BufRaw<16> {
+    typedef unsigned int type __attribute__((ext_vector_type(4)));
+    template <unsigned CP = 0> static __device__ __forceinline__ type ld(__amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { return __builtin_amdgcn_raw_buffer_load_b128(r, v, s, CP); }
+    template <unsigned CP = 0> static __device__ __forceinline__ void st(type d, __amdgpu_buffer_rsrc_t r, unsigned v, unsigned s) { __builtin_amdgcn_raw_buffer_store_b128(d, r, v, s, CP); }
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 #endif

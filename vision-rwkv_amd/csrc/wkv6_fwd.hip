@@ -27,7 +27,7 @@ int validate(int B, int T, int C, int H, int rkv_dtype, int w_dtype) {
         set_error("wkv6_fwd: w must be fp32 or have the dtype of r, k, v");
         return VRWKV_UNSUPPORTED_DTYPE;
     }
-    if ((long long)B * T * C >= (1LL << 40) || (long long)B * H > 0x7fffffffLL) {
+    if ((long long)B * T * C >= (1LL << 40) || (long long)B * H > 0x7fffffffLL || (long long)T * C >= (1LL << 29)) {
         set_error("wkv6_fwd: tensor too large");
         return VRWKV_UNSUPPORTED_SHAPE;
     }
@@ -36,42 +36,37 @@ int validate(int B, int T, int C, int H, int rkv_dtype, int w_dtype) {
 
 template <typename IO, typename WT>
 int launch_scalar(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
-                  const unsigned char* todo, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
+                  int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
     const dim3 grid(B * H), block(256);
     const IO* rr = static_cast<const IO*>(r);
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
     const WT* ww = static_cast<const WT*>(w);
     if (w_is_ew) {
-        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
     } else {
-        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 1, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_scalar_kernel<IO, WT, 0, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
     }
     return check_launch("wkv6_fwd");
 }
 
-// Chunked matrix-core passes (descending, then ascending), then the exact kernel for whatever
-// sequences they flagged as out of range.
+// One launch: both passes of a (b,h) sequence side by side in one workgroup, out-of-range sequences
+// redone in place by the sequential recurrence.
 template <typename IO, typename WT>
 int launch_chunked(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
-                   unsigned char* todo, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
-    const dim3 grid(B * H), block(128);
+                   int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
+    const dim3 grid(B * H), block(256);
     const IO* rr = static_cast<const IO*>(r);
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
     const WT* ww = static_cast<const WT*>(w);
-    if (w_is_ew) {
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 1, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 0, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-    } else {
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 1, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, 0, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, todo, T, C, H);
-    }
-    const int rc = check_launch("wkv6_fwd (chunked)");
-    if (rc != VRWKV_OK) return rc;
-    return launch_scalar<IO, WT>(r, k, v, w, u, y, todo, B, T, C, H, w_is_ew, st);
+    if (w_is_ew)
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+    else
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+    return check_launch("wkv6_fwd (chunked)");
 }
 
 bool force_scalar() {
@@ -82,16 +77,16 @@ bool force_scalar() {
 template <typename IO, typename WT>
 int launch_any(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
                void* ws, int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
-    if (force_scalar()) return launch_scalar<IO, WT>(r, k, v, w, u, y, nullptr, B, T, C, H, w_is_ew, st);
-    return launch_chunked<IO, WT>(r, k, v, w, u, y, static_cast<unsigned char*>(ws), B, T, C, H, w_is_ew, st);
+    (void)ws;
+    if (force_scalar()) return launch_scalar<IO, WT>(r, k, v, w, u, y, B, T, C, H, w_is_ew, st);
+    return launch_chunked<IO, WT>(r, k, v, w, u, y, B, T, C, H, w_is_ew, st);
 }
 
 }  // namespace
 
 extern "C" size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H) {
-    (void)T; (void)C;
-    if (B <= 0 || H <= 0) return 0;
-    return ((size_t)2 * B * H + 255) & ~(size_t)255;     // one "left to the exact kernel" flag per pass and sequence
+    (void)B; (void)T; (void)C; (void)H;
+    return 0;                                            // no workspace is needed (kept for ABI symmetry)
 }
 
 extern "C" int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, const float* u,
@@ -99,11 +94,7 @@ extern "C" int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const
                               void* workspace, size_t workspace_bytes, void* hip_stream) {
     int rc = validate(B, T, C, H, rkv_dtype, w_dtype);
     if (rc != VRWKV_OK) return rc;
-    if (!force_scalar() && (!workspace || workspace_bytes < (size_t)2 * B * H)) {
-        set_error("wkv6_fwd: workspace of %zu bytes required (got %zu)", (size_t)2 * B * H,
-                  workspace ? workspace_bytes : (size_t)0);
-        return VRWKV_WORKSPACE_TOO_SMALL;
-    }
+    (void)workspace_bytes;
     if (!r || !k || !v || !w || !u || !y) {
         set_error("wkv6_fwd: null pointer argument");
         return VRWKV_INVALID_ARG;

@@ -2,15 +2,17 @@
 //
 // Bidirectional RWKV-6 scan of
 // classification/mmcls_custom/models/backbones/cuda_v6/wkv6_cuda.cu:6-97, evaluated as two
-// passes (DIR 1: tokens descending, writes y; DIR 0: ascending with the bonus u, adds to y),
-// each pass being the same causal algorithm on its own token order n = 0..T-1:
+// passes (descending; ascending with the bonus u), each the same causal algorithm on its own
+// token order n = 0..T-1:
 //
 //   y_n = sum_j r_n[j] ( u[j] k_n[j] v_n  +  sum_{m<n} (prod_{m<l<n} d_l[j]) k_m[j] v_m )
 //
+// One 256-thread workgroup per (b,h): waves 0,1 run the descending pass, waves 2,3 the ascending
+// one, side by side and in lockstep (chunk step s of both passes between the same barriers).
 // Chunks of 32 tokens.  With the in-chunk cumulative log-decay P_n = sum_{l<=n} log d_l
 // (Pex_n = P_n - log d_n) and the mid-chunk reference Pref = P_15:
 //   rt_n = r_n * exp(Pex_n - Pref),   kt_m = k_m * exp(Pref - P_m)      (rt_n . kt_m = decay for m<n)
-//   A[n][m] = rt_n . kt_m  (m < n),  0 otherwise                          -> MFMA 1
+//   A[n][m] = rt_n . kt_m  (m < n),  bonus_n = (r_n u) . k_n  (m = n, ascending pass), 0 otherwise -> MFMA 1
 //   Y       = A V  +  rt (diag(e^Pref) S)                                 -> MFMA 2, 3
 //   S'      = diag(e^P31) S + diag(e^(P31-Pref)) (kt^T V)                 -> MFMA 4
 // S (64x64 fp32) never leaves the accumulator registers: each wave owns the 32 value columns of
@@ -18,16 +20,22 @@
 // is taken in the order the accumulator layout provides, and the A operand is read from LDS in
 // that same order); likewise A goes from the accumulators of MFMA 1 into the A operand of MFMA 2.
 //
+// y: every token is reached once by each pass.  The pass that reaches it at the earlier chunk step
+// stores, the other one adds at its (later) step, after the barrier that ends every step (on a tie the
+// descending pass stores before that barrier and the ascending pass adds after it) -- y is never
+// zero-filled, and there is no second launch.
+//
 // Precision: every operand that is computed rather than loaded (rt, kt, A, S) is split into a
 // bf16 head and a bf16 tail and the products head*head + head*tail + tail*head are accumulated,
 // which keeps the result within ~3e-5 of the fp32 recurrence (one bf16 rounding of any of them
 // alone costs ~1e-2).  v is exact in bf16 for bf16 input and split in two for fp16 / fp32 input.
 //
 // Range: the factorisation needs |P31| <= 60 in every chunk (decay over 32 tokens no stronger
-// than e^-60).  A (b,h) sequence with a chunk outside that range is left to the sequential-state
-// kernel: the pass records it in `todo` and stops.
+// than e^-60).  A (b,h) sequence with a chunk outside that range is redone from scratch by the same
+// workgroup with the sequential-state recurrence.
 #pragma once
 #include "vrwkv_common.h"
+#include "wkv6_fwd_scalar.h"
 #include <type_traits>
 
 namespace vrwkv {
@@ -47,20 +55,6 @@ constexpr float SAFE_DECAY = 60.f;
 __device__ __forceinline__ bf16x8 cat8(bf16x4 a, bf16x4 b) {
     return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
-// Sum over the 64 lanes, result wave-uniform: four DPP steps inside each 16-lane row (VALU rate),
-// then the four row sums through scalar registers.
-__device__ __forceinline__ float wave_sum(float x) {
-    auto dpp = [](float v, auto ctrl) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
-    };
-    x += dpp(x, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
-    x += dpp(x, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
-    x += dpp(x, std::integral_constant<int, 0x141>{});   // row_half_mirror
-    x += dpp(x, std::integral_constant<int, 0x140>{});   // row_mirror
-    const int xi = __builtin_bit_cast(int, x);
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
-}
 // head/tail split of eight fp32 accumulator values into two packed bf16 operands
 __device__ __forceinline__ void split8(const float (&x)[8], bf16x8& hi, bf16x8& lo) {
 #pragma unroll
@@ -71,65 +65,145 @@ __device__ __forceinline__ void split8(const float (&x)[8], bf16x8& hi, bf16x8& 
     }
 }
 
-// VSPLIT: v is given in a type that is not exact in bf16 (fp16, fp32) and is split in two.
-template <typename IO, typename WT, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(128)
+// DPP move: lane reads `v` of the lane selected by CTRL (0 where there is none).
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// 16 values per lane -> per 16-lane row, the row sums of all 16: lane l ends up with the sum over
+// its row of value index 8*(l&1) + 4*((l>>1)&1) + 2*((l>>3)&1) + ((l>>2)&1).  Transposing butterfly:
+// at each step a lane keeps one half of its values and hands the other half to its partner.
+__device__ __forceinline__ float row_sums16(const float (&p)[16], int lane, int& index) {
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
+    float a8[8], a4[4], a2[2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a8[i] = (b0 ? p[8 + i] : p[i]) + dpp_get<0xB1>(b0 ? p[i] : p[8 + i]);     // quad_perm [1,0,3,2]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a4[i] = (b1 ? a8[4 + i] : a8[i]) + dpp_get<0x4E>(b1 ? a8[i] : a8[4 + i]); // quad_perm [2,3,0,1]
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a2[i] = (b3 ? a4[2 + i] : a4[i]) + dpp_get<0x128>(b3 ? a4[i] : a4[2 + i]); // row_ror:8
+    const float give = b2 ? a2[0] : a2[1];
+    const float from_lo = dpp_get<0x114>(give), from_hi = dpp_get<0x104>(give);   // row_shr:4 (from l-4), row_shl:4 (from l+4)
+    const float recv = b2 ? from_lo : from_hi;                            // both moves run with every lane active
+    index = (b0 ? 8 : 0) + (b1 ? 4 : 0) + (b3 ? 2 : 0) + (b2 ? 1 : 0);
+    return (b2 ? a2[1] : a2[0]) + recv;
+}
+
+// Per-pass LDS operands.  VSPLIT: v is given in a type that is not exact in bf16 (fp16, fp32) and is split in two.
+template <bool VSPLIT>
+struct __attribute__((aligned(16))) PassLds {
+    __bf16 Rh[LC][PJ], Rl[LC][PJ], Kh[LC][PJ], Kl[LC][PJ];
+    __bf16 Kth[HN][PS], Ktl[HN][PS], Vt[HN][PS], Vtl[VSPLIT ? HN : 1][PS];
+    float C1[HN], C2[HN], C3[HN], Tot[HN], Bon[4][LC];
+};
+
+template <typename IO, typename WT, bool W_IS_EW>
+__global__ __launch_bounds__(256, 2)
 void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
                            const WT* __restrict__ w_, const float* __restrict__ u_, float* __restrict__ y_,
-                           unsigned char* __restrict__ todo, int T, int C, int H)
+                           int T, int C, int H)
 {
     constexpr bool VSPLIT = !(sizeof(IO) == 2 && __is_same(IO, __hip_bfloat16));
-    __shared__ __attribute__((aligned(16))) __bf16 sRh[LC][PJ], sRl[LC][PJ], sKh[LC][PJ], sKl[LC][PJ];
-    __shared__ __attribute__((aligned(16))) __bf16 sKth[HN][PS], sKtl[HN][PS], sVt[HN][PS], sVtl[VSPLIT ? HN : 1][PS];
-    __shared__ __attribute__((aligned(16))) float sC1[HN], sC2[HN], sC3[HN], sTot[HN], sBonus[LC];
+    __shared__ PassLds<VSPLIT> lds[2];
     __shared__ int sFlag;
+    static_assert(sizeof(PassLds<VSPLIT>) * 2 >= 4 * 2 * 3 * N * sizeof(float), "fallback staging must fit");
 
     const int lane = threadIdx.x & 63;
-    const int q = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);    // wave: token half in stage E, value half in stage M
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = wave & 1;                      // token half in stage E, value half in stage M
+    const bool asc = wave >= 2;                  // waves 2,3: ascending pass (with the bonus)
+    PassLds<VSPLIT>& L = lds[asc ? 1 : 0];
     const int g = lane >> 5, x = lane & 31;
     const int bh = blockIdx.x;
     const int b = bh / H, h = bh % H;
     const size_t base = (size_t)b * T * C + (size_t)h * HN;
     const int nchunk = (T + LC - 1) / LC;
-    const float uj = DIR == 0 ? u_[h * HN + lane] : 0.f;
+    const float uj = asc ? u_[h * HN + lane] : 0.f;
     if (threadIdx.x == 0) sFlag = 0;
+    __syncthreads();
 
     f32x16 S0 = {0}, S1 = {0};          // state tiles: rows j = 32*jh + 8(r/4)+4g+(r%4), column i = 32q + x
+    bool bail = false;
 
-    for (int ch = 0; ch < nchunk; ++ch) {
-        // =============================== stage E: elementwise =================================
-        // wave q prepares tokens n = 16q .. 16q+15 of the chunk; lane = channel j (and i for v)
-        float rr[16], kk[16], vv[16], ld[16];
+    // The decay rows of a chunk are fetched one step ahead (when the previous step enters its matrix stage),
+    // so the cumulative decay can start at once; r, k, v follow at the top of the step and are needed only
+    // after the first barrier.
+    using RawIO = typename BufRaw<sizeof(IO)>::type;
+    using RawW = typename BufRaw<sizeof(WT)>::type;
+    // descriptors over this (b,h)'s 64-channel column block of the batch slab; token rows are C elements apart
+    const unsigned span_io = (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(IO));
+    const unsigned span_w = (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(WT));
+    const __amdgpu_buffer_rsrc_t rsr = make_rsrc(r_ + base, span_io), rsk = make_rsrc(k_ + base, span_io),
+                                 rsv = make_rsrc(v_ + base, span_io), rsw = make_rsrc(w_ + base, span_w),
+                                 rsy = make_rsrc(y_ + base, (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(float)));
+    RawIO rraw[16], kraw[16], vraw[16];
+    RawW wraw[16];
+    auto fetch_w = [&](int ch) {
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
             const int ng = ch * LC + 16 * q + m;
-            const bool ok = ng < T;
-            const int t = DIR == 0 ? ng : T - 1 - ng;
-            const size_t o = base + (size_t)(ok ? t : 0) * C + lane;
-            const float fr = to_f32(r_[o]), fk = to_f32(k_[o]), fv = to_f32(v_[o]), fw = to_f32(w_[o]);
-            rr[m] = ok ? fr : 0.f;
-            kk[m] = ok ? fk : 0.f;
-            vv[m] = ok ? fv : 0.f;
+            const int t = ng < T ? (asc ? ng : T - 1 - ng) : 0;           // wave-uniform: a scalar row offset
+            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)t * C * (unsigned)sizeof(WT));
+        }
+    };
+    auto fetch_rkv = [&](int ch) {
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const int ng = ch * LC + 16 * q + m;
+            const int t = ng < T ? (asc ? ng : T - 1 - ng) : 0;
+            const unsigned so = (unsigned)t * C * (unsigned)sizeof(IO), vo = lane * (unsigned)sizeof(IO);
+            rraw[m] = BufRaw<sizeof(IO)>::ld(rsr, vo, so);
+            kraw[m] = BufRaw<sizeof(IO)>::ld(rsk, vo, so);
+            vraw[m] = BufRaw<sizeof(IO)>::ld(rsv, vo, so);
+        }
+    };
+    auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
+    auto cvtw = [](RawW raw) { WT t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
+    // byte offset of y[t][icol] for this lane's accumulator register r at chunk step ch (OOB when past T)
+    auto y_off = [&](int ch, int r, int icol) -> unsigned {
+        const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
+        const int t = asc ? ng : T - 1 - ng;
+        return ng < T ? (unsigned)(((size_t)t * C + icol) * sizeof(float)) : OOB_OFFSET;
+    };
+    fetch_w(0);
+
+    for (int ch = 0; ch < nchunk; ++ch) {
+        // =============================== stage E: elementwise =================================
+        // wave q of the pass prepares tokens n = 16q .. 16q+15 of the chunk; lane = channel j (and i for v)
+        fetch_rkv(ch);                                                   // used after the first barrier
+        float ld[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const bool ok = ch * LC + 16 * q + m < T;
+            const float fw = cvtw(wraw[m]);
             ld[m] = ok ? (W_IS_EW ? fw : -__expf(fw)) : 0.f;
         }
         float p[16];
         p[0] = ld[0];
 #pragma unroll
         for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
-        if (q == 0) sTot[lane] = p[15];
+        if (q == 0) L.Tot[lane] = p[15];
         lds_barrier();                                                   // (1)
-        const float pref = sTot[lane];                                   // P_15
+        const float pref = L.Tot[lane];                                  // P_15
         const float off = q == 1 ? pref : 0.f;
         if (q == 1) {
             const float p31 = p[15] + off;
-            sC2[lane] = __expf(p31);
-            sC3[lane] = __expf(p31 - pref);
+            L.C2[lane] = __expf(p31);
+            L.C3[lane] = __expf(p31 - pref);
             if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY)) != 0ull && lane == 0) sFlag = 1;
         } else {
-            sC1[lane] = __expf(pref);
+            L.C1[lane] = __expf(pref);
         }
         {
             bf16x8 kth[2], ktl[2], vth[2], vtl[2];
+            float rr[16], kk[16], vv[16];
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                const bool ok = ch * LC + 16 * q + m < T;
+                rr[m] = ok ? cvt(rraw[m]) : 0.f;
+                kk[m] = ok ? cvt(kraw[m]) : 0.f;
+                vv[m] = ok ? cvt(vraw[m]) : 0.f;
+            }
 #pragma unroll
             for (int m = 0; m < 16; ++m) {
                 const int n = 16 * q + m;
@@ -139,45 +213,59 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 const float rt = rr[m] * f1, kt = kk[m] * f2;
                 const __bf16 rh = (__bf16)rt, kh = (__bf16)kt;
                 const __bf16 rl = (__bf16)(rt - (float)rh), kl = (__bf16)(kt - (float)kh);
-                sRh[n][lane] = rh; sRl[n][lane] = rl;
-                sKh[n][lane] = kh; sKl[n][lane] = kl;
+                L.Rh[n][lane] = rh; L.Rl[n][lane] = rl;
+                L.Kh[n][lane] = kh; L.Kl[n][lane] = kl;
                 kth[m >> 3][m & 7] = kh; ktl[m >> 3][m & 7] = kl;
                 const __bf16 vh = (__bf16)vv[m];
                 vth[m >> 3][m & 7] = vh;
                 if (VSPLIT) vtl[m >> 3][m & 7] = (__bf16)(vv[m] - (float)vh);
-                if (DIR == 0) {
-                    const float c = wave_sum(rr[m] * uj * kk[m]);
-                    if (lane == 0) sBonus[n] = c;
-                }
             }
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                *reinterpret_cast<bf16x8*>(&sKth[lane][16 * q + 8 * e]) = kth[e];
-                *reinterpret_cast<bf16x8*>(&sKtl[lane][16 * q + 8 * e]) = ktl[e];
-                *reinterpret_cast<bf16x8*>(&sVt[lane][16 * q + 8 * e]) = vth[e];
-                if (VSPLIT) *reinterpret_cast<bf16x8*>(&sVtl[lane][16 * q + 8 * e]) = vtl[e];
+                *reinterpret_cast<bf16x8*>(&L.Kth[lane][16 * q + 8 * e]) = kth[e];
+                *reinterpret_cast<bf16x8*>(&L.Ktl[lane][16 * q + 8 * e]) = ktl[e];
+                *reinterpret_cast<bf16x8*>(&L.Vt[lane][16 * q + 8 * e]) = vth[e];
+                if (VSPLIT) *reinterpret_cast<bf16x8*>(&L.Vtl[lane][16 * q + 8 * e]) = vtl[e];
+            }
+            if (asc) {                                                    // bonus_n = sum_j r_n[j] u[j] k_n[j]
+                float pu[16];
+#pragma unroll
+                for (int m = 0; m < 16; ++m) pu[m] = rr[m] * uj * kk[m];
+                int idx;
+                const float rs = row_sums16(pu, lane, idx);
+                L.Bon[lane >> 4][16 * q + idx] = rs;                      // the four 16-channel rows are added by the reader
             }
         }
         lds_barrier();                                                   // (2)
-        if (sFlag) {                                                      // out of range: leave to the exact kernel
-            if (threadIdx.x == 0) todo[(size_t)DIR * gridDim.x + bh] = 1;
-            return;
-        }
+        if (sFlag) { bail = true; break; }                               // out of range: redo with the exact recurrence
+
+        if (ch + 1 < nchunk) fetch_w(ch + 1);                             // next chunk's decays, behind the matrix stage
 
         // ================================= stage M: matrix cores ===============================
         const int icol = 32 * q + x;                                      // value column of this lane
+        // y: lane = column i, register r = token 8(r/4)+4g+(r%4).  The other pass reaches the token with
+        // pass index ng at its chunk step (T-1-ng)/LC.  Where it was there at an earlier step, its value is
+        // in memory already (made visible by that step's closing barrier): fetch it now, behind the MFMAs.
+        float prev[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
+            const bool second = ng < T && ch > (T - 1 - ng) / LC;
+            prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, second ? y_off(ch, r, icol) : OOB_OFFSET, 0));
+        }
         // ---- MFMA 1: A^T: acc[m = s][n = t]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
         f32x16 accA = {0};
 #pragma unroll
         for (int kq = 0; kq < 4; ++kq) {
-            const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&sKh[x][16 * kq + 8 * g]);
-            const bf16x8 al = *reinterpret_cast<const bf16x8*>(&sKl[x][16 * kq + 8 * g]);
-            const bf16x8 bh_ = *reinterpret_cast<const bf16x8*>(&sRh[x][16 * kq + 8 * g]);
-            const bf16x8 bl = *reinterpret_cast<const bf16x8*>(&sRl[x][16 * kq + 8 * g]);
+            const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&L.Kh[x][16 * kq + 8 * g]);
+            const bf16x8 al = *reinterpret_cast<const bf16x8*>(&L.Kl[x][16 * kq + 8 * g]);
+            const bf16x8 bh_ = *reinterpret_cast<const bf16x8*>(&L.Rh[x][16 * kq + 8 * g]);
+            const bf16x8 bl = *reinterpret_cast<const bf16x8*>(&L.Rl[x][16 * kq + 8 * g]);
             accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh_, accA, 0, 0, 0);
             accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, accA, 0, 0, 0);
             accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh_, accA, 0, 0, 0);
         }
+        const float diag = asc ? (L.Bon[0][x] + L.Bon[1][x]) + (L.Bon[2][x] + L.Bon[3][x]) : 0.f;
         bf16x8 Ah[2], Al[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -186,7 +274,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             for (int e = 0; e < 8; ++e) {
                 const int r = 8 * ks + e;
                 const int s = 8 * (r / 4) + 4 * g + (r % 4);
-                a8[e] = s < x ? accA[r] : 0.f;                            // strictly earlier tokens only
+                a8[e] = s < x ? accA[r] : (s == x ? diag : 0.f);          // earlier tokens; the token itself through the bonus
             }
             split8(a8, Ah[ks], Al[ks]);
         }
@@ -194,13 +282,13 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         f32x16 accY = {0};
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const bf16x8 bv = cat8(*reinterpret_cast<const bf16x4*>(&sVt[icol][16 * ks + 4 * g]),
-                                   *reinterpret_cast<const bf16x4*>(&sVt[icol][16 * ks + 8 + 4 * g]));
+            const bf16x8 bv = cat8(*reinterpret_cast<const bf16x4*>(&L.Vt[icol][16 * ks + 4 * g]),
+                                   *reinterpret_cast<const bf16x4*>(&L.Vt[icol][16 * ks + 8 + 4 * g]));
             accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ah[ks], bv, accY, 0, 0, 0);
             accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Al[ks], bv, accY, 0, 0, 0);
             if (VSPLIT) {
-                const bf16x8 bvl = cat8(*reinterpret_cast<const bf16x4*>(&sVtl[icol][16 * ks + 4 * g]),
-                                        *reinterpret_cast<const bf16x4*>(&sVtl[icol][16 * ks + 8 + 4 * g]));
+                const bf16x8 bvl = cat8(*reinterpret_cast<const bf16x4*>(&L.Vtl[icol][16 * ks + 4 * g]),
+                                        *reinterpret_cast<const bf16x4*>(&L.Vtl[icol][16 * ks + 8 + 4 * g]));
                 accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ah[ks], bvl, accY, 0, 0, 0);
             }
         }
@@ -213,17 +301,17 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 float s8[8];
 #pragma unroll
                 for (int e4 = 0; e4 < 2; ++e4) {
-                    const f32x4 c1 = *reinterpret_cast<const f32x4*>(&sC1[32 * jh + 16 * ks + 8 * e4 + 4 * g]);
+                    const f32x4 c1 = *reinterpret_cast<const f32x4*>(&L.C1[32 * jh + 16 * ks + 8 * e4 + 4 * g]);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) s8[4 * e4 + e] = S[8 * ks + 4 * e4 + e] * c1[e];
                 }
                 bf16x8 sh, sl;
                 split8(s8, sh, sl);
                 const int j0 = 32 * jh + 16 * ks + 4 * g;
-                const bf16x8 ah = cat8(*reinterpret_cast<const bf16x4*>(&sRh[x][j0]),
-                                       *reinterpret_cast<const bf16x4*>(&sRh[x][j0 + 8]));
-                const bf16x8 al = cat8(*reinterpret_cast<const bf16x4*>(&sRl[x][j0]),
-                                       *reinterpret_cast<const bf16x4*>(&sRl[x][j0 + 8]));
+                const bf16x8 ah = cat8(*reinterpret_cast<const bf16x4*>(&L.Rh[x][j0]),
+                                       *reinterpret_cast<const bf16x4*>(&L.Rh[x][j0 + 8]));
+                const bf16x8 al = cat8(*reinterpret_cast<const bf16x4*>(&L.Rl[x][j0]),
+                                       *reinterpret_cast<const bf16x4*>(&L.Rl[x][j0 + 8]));
                 accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, sh, accY, 0, 0, 0);
                 accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, sl, accY, 0, 0, 0);
                 accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, sh, accY, 0, 0, 0);
@@ -235,55 +323,67 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             f32x16 accM = {0};
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&sKth[32 * jh + x][16 * ks + 8 * g]);
-                const bf16x8 al = *reinterpret_cast<const bf16x8*>(&sKtl[32 * jh + x][16 * ks + 8 * g]);
-                const bf16x8 bv = *reinterpret_cast<const bf16x8*>(&sVt[icol][16 * ks + 8 * g]);
+                const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&L.Kth[32 * jh + x][16 * ks + 8 * g]);
+                const bf16x8 al = *reinterpret_cast<const bf16x8*>(&L.Ktl[32 * jh + x][16 * ks + 8 * g]);
+                const bf16x8 bv = *reinterpret_cast<const bf16x8*>(&L.Vt[icol][16 * ks + 8 * g]);
                 accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bv, accM, 0, 0, 0);
                 accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bv, accM, 0, 0, 0);
                 if (VSPLIT) {
-                    const bf16x8 bvl = *reinterpret_cast<const bf16x8*>(&sVtl[icol][16 * ks + 8 * g]);
+                    const bf16x8 bvl = *reinterpret_cast<const bf16x8*>(&L.Vtl[icol][16 * ks + 8 * g]);
                     accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bvl, accM, 0, 0, 0);
                 }
             }
             f32x16& S = jh == 0 ? S0 : S1;
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const f32x4 c2 = *reinterpret_cast<const f32x4*>(&sC2[32 * jh + 8 * r4 + 4 * g]);
-                const f32x4 c3 = *reinterpret_cast<const f32x4*>(&sC3[32 * jh + 8 * r4 + 4 * g]);
+                const f32x4 c2 = *reinterpret_cast<const f32x4*>(&L.C2[32 * jh + 8 * r4 + 4 * g]);
+                const f32x4 c3 = *reinterpret_cast<const f32x4*>(&L.C3[32 * jh + 8 * r4 + 4 * g]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + c3[e] * accM[4 * r4 + e];
             }
         }
-        // ---- bonus (ascending pass) and store: lane = column i, register r = token 8(r/4)+4g+(r%4) ----
+        // ---- y: store where this pass is first (on a tie: the descending pass),
+        //      store the sum where the other pass was first; the ascending pass adds its tie tokens after
+        //      the barrier ----
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const int n0 = 8 * r4 + 4 * g;
-            f32x4 bon = {0.f, 0.f, 0.f, 0.f};
-            if (DIR == 0) {
-                const f32x4 c = *reinterpret_cast<const f32x4*>(&sBonus[n0]);
-                const bf16x4 vh = *reinterpret_cast<const bf16x4*>(&sVt[icol][n0]);
+        for (int r = 0; r < 16; ++r) {
+            const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
+            const bool mine = ch != (T - 1 - ng) / LC || !asc;
+            BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, mine ? y_off(ch, r, icol) : OOB_OFFSET, 0);
+        }
+        // end of the step: every LDS read of this chunk is done, and the stores above become visible
+        // to the other pass of this workgroup
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();                                    // (3)
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const int rem = T - 1 - ch * LC;                                  // other-pass index of this chunk's first token
+        if (asc && (ch == rem / LC || (rem >= LC - 1 && ch == (rem - (LC - 1)) / LC))) {   // wave-uniform: tie tokens here
 #pragma unroll
-                for (int e = 0; e < 4; ++e) bon[e] = c[e] * (float)vh[e];
-                if (VSPLIT) {
-                    const bf16x4 vl = *reinterpret_cast<const bf16x4*>(&sVtl[icol][n0]);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) bon[e] += c[e] * (float)vl[e];
-                }
+            for (int r = 0; r < 16; ++r) {
+                const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
+                prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, ch == (T - 1 - ng) / LC ? y_off(ch, r, icol) : OOB_OFFSET, 0));
             }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int ng = ch * LC + n0 + e;
-                if (ng < T) {
-                    const int t = DIR == 0 ? ng : T - 1 - ng;
-                    float* yp = y_ + base + (size_t)t * C + icol;
-                    const float val = accY[4 * r4 + e] + bon[e];
-                    if (DIR == 0) *yp += val; else *yp = val;
-                }
+            for (int r = 0; r < 16; ++r) {
+                const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, ch == (T - 1 - ng) / LC ? y_off(ch, r, icol) : OOB_OFFSET, 0);
             }
         }
-        lds_barrier();                                                   // (3) LDS is rewritten by the next chunk
     }
-    if (threadIdx.x == 0) todo[(size_t)DIR * gridDim.x + bh] = 0;
+
+    if (bail) {
+        // Some chunk decays faster than the factorisation can represent: recompute the whole sequence
+        // with the sequential recurrence (it rewrites every y of this (b,h)).
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        float* stage = reinterpret_cast<float*>(&lds[0]);
+        wkv6_scalar_pass<IO, WT, 1, W_IS_EW>(r_, k_, v_, w_, u_, y_, stage, bh, T, C, H);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        wkv6_scalar_pass<IO, WT, 0, W_IS_EW>(r_, k_, v_, w_, u_, y_, stage, bh, T, C, H);
+    }
 }
 
 }  // namespace wkv6_detail

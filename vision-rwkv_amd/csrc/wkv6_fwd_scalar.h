@@ -18,19 +18,18 @@ namespace wkv6_detail {
 
 constexpr int N = 64;            // head size (vrwkv6.py:23)
 
-// DIR 0: ascending pass with the bonus, accumulates into y.  DIR 1: descending pass, writes y.
+// One pass over one (b,h) sequence by a 256-thread workgroup.  DIR 0: ascending pass with the bonus,
+// accumulates into y.  DIR 1: descending pass, writes y.  s_row: 4*2*3*64 floats of LDS.
 template <typename IO, typename WT, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(256)
-void wkv6_fwd_scalar_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
-                            const WT* __restrict__ w_, const float* __restrict__ u_, float* __restrict__ y_,
-                            const unsigned char* __restrict__ todo, int T, int C, int H)
+__device__ __forceinline__
+void wkv6_scalar_pass(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
+                      const WT* __restrict__ w_, const float* __restrict__ u_, float* __restrict__ y_,
+                      float* __restrict__ s_row_raw, int bh, int T, int C, int H)
 {
-    // `todo` (one flag per pass and sequence) marks what the chunked kernel left undone
-    if (todo && !(todo[blockIdx.x] | todo[gridDim.x + blockIdx.x])) return;
-    __shared__ __attribute__((aligned(16))) float s_row[4][2][3][N];   // [wave][buffer][r,k,d][j]
+    float (*s_row)[2][3][N] = reinterpret_cast<float (*)[2][3][N]>(s_row_raw);   // [wave][buffer][r,k,d][j]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int b = bh / H, h = bh % H;
     const int jg = lane & 3;                             // which 16 key channels
     const int i = wave * 16 + (lane >> 2);               // value channel
     const size_t base = (size_t)b * T * C + (size_t)h * N;
@@ -86,6 +85,16 @@ void wkv6_fwd_scalar_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_
         }
         buf ^= 1;
     }
+}
+
+template <typename IO, typename WT, int DIR, bool W_IS_EW>
+__global__ __launch_bounds__(256)
+void wkv6_fwd_scalar_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
+                            const WT* __restrict__ w_, const float* __restrict__ u_, float* __restrict__ y_,
+                            int T, int C, int H)
+{
+    __shared__ __attribute__((aligned(16))) float s_row[4 * 2 * 3 * N];
+    wkv6_scalar_pass<IO, WT, DIR, W_IS_EW>(r_, k_, v_, w_, u_, y_, s_row, blockIdx.x, T, C, H);
 }
 
 }  // namespace wkv6_detail
