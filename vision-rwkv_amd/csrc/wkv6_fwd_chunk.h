@@ -20,10 +20,10 @@
 // is taken in the order the accumulator layout provides, and the A operand is read from LDS in
 // that same order); likewise A goes from the accumulators of MFMA 1 into the A operand of MFMA 2.
 //
-// y: every token is reached once by each pass.  The pass that reaches it at the earlier chunk step
-// stores, the other one adds at its (later) step, after the barrier that ends every step (on a tie the
-// descending pass stores before that barrier and the ascending pass adds after it) -- y is never
-// zero-filled, and there is no second launch.
+// y: both passes walk the same chunk grid from opposite ends.  The pass that reaches a chunk at the
+// earlier step stores, the other one adds at its (later) step, after the barrier that ends every step (at
+// the middle chunk of an odd count the descending pass stores before that barrier and the ascending pass
+// adds after it) -- y is never zero-filled, and there is no second launch.
 //
 // Precision: every operand that is computed rather than loaded (rt, kt, A, S) is split into a
 // bf16 head and a bf16 tail and the products head*head + head*tail + tail*head are accumulated,
@@ -37,6 +37,10 @@
 #include "vrwkv_common.h"
 #include "wkv6_fwd_scalar.h"
 #include <type_traits>
+
+#ifndef WKV6_STAMP
+#define WKV6_STAMP(phase)                 // timing hook of the micro-benchmarks; nothing in the library build
+#endif
 
 namespace vrwkv {
 namespace wkv6_detail {
@@ -138,20 +142,26 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                                  rsy = make_rsrc(y_ + base, (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(float)));
     RawIO rraw[16], kraw[16], vraw[16];
     RawW wraw[16];
+    // Both passes walk the same 32-token chunks of the token axis (the ascending pass chunk 0, 1, ..., the
+    // descending pass chunk nchunk-1, ..., 0), so everything that depends on the position is wave-uniform.
+    // Pass index n = 0..31 inside a chunk is token 32c + n (ascending) or 32c + 31 - n (descending); tokens
+    // past T (only in the last chunk; for the descending pass they come first) are r = k = v = 0, d = 1.
+    auto chunk_of = [&](int ch) { return asc ? ch : nchunk - 1 - ch; };
+    auto token_of = [&](int c, int n) { return c * LC + (asc ? n : LC - 1 - n); };
     auto fetch_w = [&](int ch) {
+        const int c = chunk_of(ch);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const int ng = ch * LC + 16 * q + m;
-            const int t = ng < T ? (asc ? ng : T - 1 - ng) : 0;           // wave-uniform: a scalar row offset
-            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)t * C * (unsigned)sizeof(WT));
+            const int t = token_of(c, 16 * q + m);                        // wave-uniform: a scalar row offset
+            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(WT));
         }
     };
     auto fetch_rkv = [&](int ch) {
+        const int c = chunk_of(ch);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const int ng = ch * LC + 16 * q + m;
-            const int t = ng < T ? (asc ? ng : T - 1 - ng) : 0;
-            const unsigned so = (unsigned)t * C * (unsigned)sizeof(IO), vo = lane * (unsigned)sizeof(IO);
+            const int t = token_of(c, 16 * q + m);
+            const unsigned so = (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(IO), vo = lane * (unsigned)sizeof(IO);
             rraw[m] = BufRaw<sizeof(IO)>::ld(rsr, vo, so);
             kraw[m] = BufRaw<sizeof(IO)>::ld(rsk, vo, so);
             vraw[m] = BufRaw<sizeof(IO)>::ld(rsv, vo, so);
@@ -159,22 +169,24 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     };
     auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
     auto cvtw = [](RawW raw) { WT t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
-    // byte offset of y[t][icol] for this lane's accumulator register r at chunk step ch (OOB when past T)
-    auto y_off = [&](int ch, int r, int icol) -> unsigned {
-        const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
-        const int t = asc ? ng : T - 1 - ng;
-        return ng < T ? (unsigned)(((size_t)t * C + icol) * sizeof(float)) : OOB_OFFSET;
+    // y[t][icol] of accumulator register r (pass index n = 8(r/4) + 4g + (r%4)): a per-lane byte offset plus a
+    // wave-uniform one; rows past T fall outside the descriptor and are dropped by the hardware.
+    const unsigned y_lane = (unsigned)(((asc ? 4 * g : 4 * (1 - g)) * C + 32 * q + x) * sizeof(float));
+    auto y_off = [&](int c, int r) -> unsigned {
+        const int nl = asc ? 8 * (r / 4) + (r % 4) : 8 * (3 - r / 4) + (3 - r % 4);
+        return y_lane + (unsigned)(c * LC + nl) * C * (unsigned)sizeof(float);
     };
     fetch_w(0);
 
     for (int ch = 0; ch < nchunk; ++ch) {
         // =============================== stage E: elementwise =================================
         // wave q of the pass prepares tokens n = 16q .. 16q+15 of the chunk; lane = channel j (and i for v)
+        WKV6_STAMP(0);
         fetch_rkv(ch);                                                   // used after the first barrier
         float ld[16];
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const bool ok = ch * LC + 16 * q + m < T;
+            const bool ok = token_of(chunk_of(ch), 16 * q + m) < T;
             const float fw = cvtw(wraw[m]);
             ld[m] = ok ? (W_IS_EW ? fw : -__expf(fw)) : 0.f;
         }
@@ -183,7 +195,9 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
 #pragma unroll
         for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
         if (q == 0) L.Tot[lane] = p[15];
+        WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
+        WKV6_STAMP(2);
         const float pref = L.Tot[lane];                                  // P_15
         const float off = q == 1 ? pref : 0.f;
         if (q == 1) {
@@ -199,7 +213,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             float rr[16], kk[16], vv[16];
 #pragma unroll
             for (int m = 0; m < 16; ++m) {
-                const bool ok = ch * LC + 16 * q + m < T;
+                const bool ok = token_of(chunk_of(ch), 16 * q + m) < T;
                 rr[m] = ok ? cvt(rraw[m]) : 0.f;
                 kk[m] = ok ? cvt(kraw[m]) : 0.f;
                 vv[m] = ok ? cvt(vraw[m]) : 0.f;
@@ -236,22 +250,25 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 L.Bon[lane >> 4][16 * q + idx] = rs;                      // the four 16-channel rows are added by the reader
             }
         }
+        WKV6_STAMP(3);
         lds_barrier();                                                   // (2)
+        WKV6_STAMP(4);
         if (sFlag) { bail = true; break; }                               // out of range: redo with the exact recurrence
 
         if (ch + 1 < nchunk) fetch_w(ch + 1);                             // next chunk's decays, behind the matrix stage
 
         // ================================= stage M: matrix cores ===============================
         const int icol = 32 * q + x;                                      // value column of this lane
-        // y: lane = column i, register r = token 8(r/4)+4g+(r%4).  The other pass reaches the token with
-        // pass index ng at its chunk step (T-1-ng)/LC.  Where it was there at an earlier step, its value is
-        // in memory already (made visible by that step's closing barrier): fetch it now, behind the MFMAs.
+        // y: the other pass reaches this chunk at step nchunk-1-ch.  If that was earlier, its values are in
+        // memory already (made visible by that step's closing barrier): fetch them now, behind the MFMAs.
+        const int cy = chunk_of(ch);
+        const bool y_second = ch > nchunk - 1 - ch, y_tie = asc && ch == nchunk - 1 - ch;     // wave-uniform
         float prev[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
-            const bool second = ng < T && ch > (T - 1 - ng) / LC;
-            prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, second ? y_off(ch, r, icol) : OOB_OFFSET, 0));
+        for (int r = 0; r < 16; ++r) prev[r] = 0.f;
+        if (y_second) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r), 0));
         }
         // ---- MFMA 1: A^T: acc[m = s][n = t]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
         f32x16 accA = {0};
@@ -342,32 +359,28 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + c3[e] * accM[4 * r4 + e];
             }
         }
-        // ---- y: store where this pass is first (on a tie: the descending pass),
-        //      store the sum where the other pass was first; the ascending pass adds its tie tokens after
-        //      the barrier ----
+        WKV6_STAMP(5);
+        // ---- y: store (sum with the other pass's value where it came first); on a tie the descending pass
+        //      stores here and the ascending pass adds after the barrier ----
+        if (!y_tie) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
-            const bool mine = ch != (T - 1 - ng) / LC || !asc;
-            BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, mine ? y_off(ch, r, icol) : OOB_OFFSET, 0);
+            for (int r = 0; r < 16; ++r)
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r), 0);
         }
         // end of the step: every LDS read of this chunk is done, and the stores above become visible
         // to the other pass of this workgroup
+        WKV6_STAMP(6);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        WKV6_STAMP(7);
         __builtin_amdgcn_s_barrier();                                    // (3)
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        const int rem = T - 1 - ch * LC;                                  // other-pass index of this chunk's first token
-        if (asc && (ch == rem / LC || (rem >= LC - 1 && ch == (rem - (LC - 1)) / LC))) {   // wave-uniform: tie tokens here
+        WKV6_STAMP(8);
+        if (y_tie) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
-                prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, ch == (T - 1 - ng) / LC ? y_off(ch, r, icol) : OOB_OFFSET, 0));
-            }
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r), 0));
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ng = ch * LC + 8 * (r / 4) + 4 * g + (r % 4);
-                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, ch == (T - 1 - ng) / LC ? y_off(ch, r, icol) : OOB_OFFSET, 0);
-            }
+            for (int r = 0; r < 16; ++r)
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r), 0);
         }
     }
 
