@@ -147,8 +147,9 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     // Pass index n = 0..31 inside a chunk is token 32c + n (ascending) or 32c + 31 - n (descending); tokens
     // past T (only in the last chunk; for the descending pass they come first) are r = k = v = 0, d = 1.
     auto chunk_of = [&](int ch) { return asc ? ch : nchunk - 1 - ch; };
-    auto token_of = [&](int c, int n) { return c * LC + (asc ? n : LC - 1 - n); };
-    auto fetch_w = [&](int ch) {
+    const int sgn = asc ? 1 : -1, n0 = asc ? 0 : LC - 1;
+    auto token_of = [&](int c, int n) { return c * LC + n0 + sgn * n; };
+    auto fetch_w = [&](int ch, int C) {
         const int c = chunk_of(ch);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
@@ -156,7 +157,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(WT));
         }
     };
-    auto fetch_rkv = [&](int ch) {
+    auto fetch_rkv = [&](int ch, int C) {
         const int c = chunk_of(ch);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
@@ -172,17 +173,21 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     // y[t][icol] of accumulator register r (pass index n = 8(r/4) + 4g + (r%4)): a per-lane byte offset plus a
     // wave-uniform one; rows past T fall outside the descriptor and are dropped by the hardware.
     const unsigned y_lane = (unsigned)(((asc ? 4 * g : 4 * (1 - g)) * C + 32 * q + x) * sizeof(float));
-    auto y_off = [&](int c, int r) -> unsigned {
-        const int nl = asc ? 8 * (r / 4) + (r % 4) : 8 * (3 - r / 4) + (3 - r % 4);
-        return y_lane + (unsigned)(c * LC + nl) * C * (unsigned)sizeof(float);
+    const int y_n0 = asc ? 0 : 27;                                        // 8(3 - r/4) + (3 - r%4) = 27 - (8(r/4) + r%4)
+    auto y_off = [&](int c, int r, int C) -> unsigned {
+        return y_lane + (unsigned)((c * LC + y_n0) * C * 4) + (unsigned)((8 * (r / 4) + (r % 4)) * (sgn * C * 4));
     };
-    fetch_w(0);
+    fetch_w(0, C);
 
     for (int ch = 0; ch < nchunk; ++ch) {
         // =============================== stage E: elementwise =================================
         // wave q of the pass prepares tokens n = 16q .. 16q+15 of the chunk; lane = channel j (and i for v)
+        // Row offsets are recomputed per step from an opaque copy of C: hoisted out of the loop they would
+        // occupy ~100 scalar registers and spill.
+        int Cs = C;
+        asm volatile("" : "+s"(Cs));
         WKV6_STAMP(0);
-        fetch_rkv(ch);                                                   // used after the first barrier
+        fetch_rkv(ch, Cs);                                                   // used after the first barrier
         float ld[16];
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
@@ -255,7 +260,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         WKV6_STAMP(4);
         if (sFlag) { bail = true; break; }                               // out of range: redo with the exact recurrence
 
-        if (ch + 1 < nchunk) fetch_w(ch + 1);                             // next chunk's decays, behind the matrix stage
+        if (ch + 1 < nchunk) fetch_w(ch + 1, Cs);                             // next chunk's decays, behind the matrix stage
 
         // ================================= stage M: matrix cores ===============================
         const int icol = 32 * q + x;                                      // value column of this lane
@@ -268,7 +273,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         for (int r = 0; r < 16; ++r) prev[r] = 0.f;
         if (y_second) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r), 0));
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r, Cs), 0));
         }
         // ---- MFMA 1: A^T: acc[m = s][n = t]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
         f32x16 accA = {0};
@@ -284,14 +289,16 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         }
         const float diag = asc ? (L.Bon[0][x] + L.Bon[1][x]) + (L.Bon[2][x] + L.Bon[3][x]) : 0.f;
         bf16x8 Ah[2], Al[2];
+        int dx = 4 * g - x;                                               // compared in place: 32 hoisted lane masks
+        asm volatile("" : "+v"(dx));                                      // would not fit the scalar registers
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             float a8[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int r = 8 * ks + e;
-                const int s = 8 * (r / 4) + 4 * g + (r % 4);
-                a8[e] = s < x ? accA[r] : (s == x ? diag : 0.f);          // earlier tokens; the token itself through the bonus
+                const int sx = 8 * (r / 4) + (r % 4) + dx;                // s - x with s = 8(r/4) + 4g + (r%4)
+                a8[e] = sx < 0 ? accA[r] : (sx == 0 ? diag : 0.f);        // earlier tokens; the token itself through the bonus
             }
             split8(a8, Ah[ks], Al[ks]);
         }
@@ -365,7 +372,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         if (!y_tie) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r), 0);
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r, Cs), 0);
         }
         // end of the step: every LDS read of this chunk is done, and the stores above become visible
         // to the other pass of this workgroup
@@ -377,10 +384,10 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         WKV6_STAMP(8);
         if (y_tie) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r), 0));
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r, Cs), 0));
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r), 0);
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r, Cs), 0);
         }
     }
 
