@@ -39,6 +39,17 @@ def test_fused_qshift_mix_against_oracle(B, Hp, Wp, C, dtype):
         assert np.array_equal(z.cpu().numpy(), xx)
 
 
+def test_patch_embedding_gemm_equals_convolution():
+    """CPU: the stem computes Conv2d(kernel = stride = patch) as one GEMM over flattened patches."""
+    import vision_rwkv_amd as ops
+    torch.manual_seed(0)
+    net = ops.VRWKV(img_size=32, embed_dims=32, depth=1)
+    img = torch.randn(2, 3, 48, 32)
+    x, res = net.embed(img)
+    want = net.patch_embed(img)
+    assert res == (3, 2) and torch.allclose(x, want.flatten(2).transpose(1, 2), atol=1e-5)
+
+
 @pytest.mark.gpu
 def test_fused_qshift_multihead_with_cls_token():
     import vision_rwkv_amd as ops

@@ -146,11 +146,31 @@ class VRWKV(nn.Module):
         if final_norm:
             self.ln1 = nn.LayerNorm(embed_dims)
 
+    def _pos_embed_for(self, res):
+        """Position embedding at grid `res`; in eval mode the interpolated table is computed once per grid
+        (the reference re-runs the bicubic resize in every forward, vrwkv.py:411-415)."""
+        if self.training or torch.is_grad_enabled():
+            return resize_pos_embed(self.pos_embed, self.patch_resolution, res, self.interpolate_mode)
+        key = (tuple(res), self.pos_embed._version, self.pos_embed.device, self.pos_embed.dtype)
+        if getattr(self, "_pos_cache_key", None) != key:
+            self._pos_cache = resize_pos_embed(self.pos_embed.detach(), self.patch_resolution, res, self.interpolate_mode)
+            self._pos_cache_key = key
+        return self._pos_cache
+
+    def embed(self, img):
+        """Patch embedding: (B, 3, H, W) -> (B, Hp*Wp, C) tokens and the patch grid (Hp, Wp)."""
+        # kernel = stride = patch: the convolution is one GEMM over the flattened patches
+        B, Cin, Hi, Wi = img.shape
+        P = self.patch_size
+        res = (Hi // P, Wi // P)
+        patches = img[:, :, :res[0] * P, :res[1] * P].reshape(B, Cin, res[0], P, res[1], P)
+        patches = patches.permute(0, 2, 4, 1, 3, 5).reshape(B, res[0] * res[1], Cin * P * P)
+        x = F.linear(patches, self.patch_embed.weight.reshape(self.patch_embed.out_channels, -1), self.patch_embed.bias)
+        return x, res
+
     def forward(self, img):
-        x = self.patch_embed(img)
-        res = (x.shape[2], x.shape[3])
-        x = x.flatten(2).transpose(1, 2)
-        x = x + resize_pos_embed(self.pos_embed, self.patch_resolution, res, self.interpolate_mode).to(x.dtype)
+        x, res = self.embed(img)
+        x = x + self._pos_embed_for(res).to(x.dtype)
         for layer in self.layers:
             x = layer(x, res)
         if self.final_norm:

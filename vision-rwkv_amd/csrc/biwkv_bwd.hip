@@ -38,16 +38,6 @@ void biwkv_bwd_serial_kernel(const float* __restrict__ w_, const float* __restri
     biwkv_bwd_serial_seq<IO>(w_, u_, k_, v_, gy_, gk_, gv_, ws, gw_part, gu_part, B, T, C, blockIdx.y, c);
 }
 
-__global__ void biwkv_bwd_reduce_kernel(const float* __restrict__ gw_part, const float* __restrict__ gu_part,
-                                        float* __restrict__ gw, float* __restrict__ gu, int B, int C)
-{
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float sw = 0.f, su = 0.f;
-    for (int b = 0; b < B; ++b) { sw += gw_part[(size_t)b * C + c]; su += gu_part[(size_t)b * C + c]; }
-    gw[c] = sw; gu[c] = su;
-}
-
 int validate(int B, int T, int C, int io_dtype) {
     if (B <= 0 || T <= 0 || C <= 0) {
         set_error("biwkv_bwd: B, T, C must be positive (got %d, %d, %d)", B, T, C);
@@ -97,7 +87,7 @@ int launch(const float* w, const float* u, const void* k, const void* v, const v
         hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
                            kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C);
     }
-    hipLaunchKernelGGL(biwkv_bwd_reduce_kernel, dim3((C + 255) / 256), dim3(256), 0, st, gw_part, gu_part, gw, gu, B, C);
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gw_part, gw, gu_part, gu, B, C);
     return check_launch("biwkv_bwd");
 }
 

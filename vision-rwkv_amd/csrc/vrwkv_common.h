@@ -92,6 +92,32 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// out[c] = sum_b part[b*C + c] for up to two (part, out) pairs (the second may be null).  256 threads =
+// 16 channels x 16 slices of the batch, so the B loads of a channel are issued 16 at a time instead of
+// one after the other; fixed summation order (deterministic).  Grid: ceil(C / 16).
+__global__ inline void batch_sum_kernel(const float* __restrict__ part0, float* __restrict__ out0,
+                                        const float* __restrict__ part1, float* __restrict__ out1, int B, int C) {
+    __shared__ float red[2][16][17];
+    const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
+    const int c = blockIdx.x * 16 + cl;
+    float s0 = 0.f, s1 = 0.f;
+    if (c < C)
+        for (int b = slice; b < B; b += 16) {
+            s0 += part0[(size_t)b * C + c];
+            if (part1) s1 += part1[(size_t)b * C + c];
+        }
+    red[0][slice][cl] = s0;
+    red[1][slice][cl] = s1;
+    __syncthreads();
+    if (slice == 0 && c < C) {
+        float t0 = 0.f, t1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { t0 += red[0][i][cl]; t1 += red[1][i][cl]; }
+        out0[c] = t0;
+        if (part1) out1[c] = t1;
+    }
+}
 #endif
 
 }  // namespace vrwkv

@@ -203,14 +203,6 @@ void wkv6_bwd_sweep_v(const IO* __restrict__ r_, const IO* __restrict__ k_,
     }
 }
 
-__global__ void wkv6_bwd_reduce_gu(const float* __restrict__ gu_part, float* __restrict__ gu, int B, int C) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float s = 0.f;
-    for (int b = 0; b < B; ++b) s += gu_part[(size_t)b * C + c];     // torch.sum(gu, 0), vrwkv6.py:69
-    gu[c] = s;
-}
-
 template <typename IO, typename WT, bool EW>
 int launch_all(const void* r, const void* k, const void* v, const void* w, const float* u, const float* gy,
                float* gr, float* gk, float* gv, float* gw, float* gu, float* ws, int B, int T, int C, int H, hipStream_t st) {
@@ -228,7 +220,7 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
     hipLaunchKernelGGL((wkv6_bwd_sweep_s<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, gr, a, gu_part, T, C, H);
     hipLaunchKernelGGL((wkv6_bwd_sweep_g<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, a, gk, gw, T, C, H);
     hipLaunchKernelGGL((wkv6_bwd_sweep_v<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, ww, u, gy, gv, T, C, H);
-    hipLaunchKernelGGL(wkv6_bwd_reduce_gu, dim3((C + 255) / 256), dim3(256), 0, st, gu_part, gu, B, C);
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gu_part, gu, (const float*)nullptr, (float*)nullptr, B, C);   // torch.sum(gu, 0), vrwkv6.py:69
     return check_launch("wkv6_bwd");
 }
 
