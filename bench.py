@@ -107,6 +107,37 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
     return out
 
 
+def backward_section(torch, ops, steps, warmup):
+    """Backward of both operators at the same VRWKV-B shapes (Bi-WKV fp32 I/O; wkv6 bf16 r,k,v, fp32 w, gy)."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(99)
+    w, u = (t.to(dev) for t in baseline_wu(torch))
+    k, v, gy = (torch.randn(B, T, C, generator=g).to(dev) for _ in range(3))
+    Hw = C // 64
+    r6, k6, v6 = (torch.randn(B, T, C, generator=g).to(dev).bfloat16() for _ in range(3))
+    w6 = (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(dev)
+    u6 = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
+    us_6 = timed(lambda: ops.wkv6_backward(B, T, C, Hw, r6, k6, v6, w6, u6, gy))
+    bytes_b = 5 * B * T * C * 4                                  # k, v, gy read; gk, gv written
+    return {"biwkv_bwd_us_per_call": round(us_b, 2), "biwkv_bwd_GBps": round(bytes_b / (us_b * 1e-6) / 1e9, 1),
+            "biwkv_bwd_pct_hbm_peak": round(100 * bytes_b / (us_b * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
+            "wkv6_bwd_us_per_call": round(us_6, 1), "wkv6_bwd_tokens_per_s": round(B * T / (us_6 * 1e-6), 1)}
+
+
 def backbone_section(torch, ops, steps, warmup):
     """VRWKV-L forward (24 blocks, C=1024, 384x384 input -> T=576) at batch 32 in bf16, random weights:
     ms per forward, and the share of it spent in the 24 Bi-WKV calls (timed alone at the same shape)."""
@@ -155,6 +186,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-wkv6", action="store_true", help="skip the secondary wkv6 measurement")
     ap.add_argument("--no-backbone", action="store_true", help="skip the VRWKV-L whole-forward measurement")
+    ap.add_argument("--no-backward", action="store_true", help="skip the backward-kernel measurements")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -256,6 +288,8 @@ def main():
         out["cpu_baseline"] = cb
     if not args.no_wkv6:
         out["wkv6"] = wkv6_section(torch, ops, max(args.steps, 10), max(args.warmup // 5, 3), not args.no_cpu_baseline)
+    if not args.no_backward:
+        out["backward"] = backward_section(torch, ops, 10, 3)
     if not args.no_backbone:
         out["backbone"] = backbone_section(torch, ops, 5, 3)
     print(json.dumps(out))

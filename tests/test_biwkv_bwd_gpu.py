@@ -116,10 +116,11 @@ def test_tiled_kernel_equals_sequential_kernel_full_size(ops, monkeypatch):
     assert gk.sum(1).abs().max().item() <= 1e-4 * gk.abs().max().item() * T ** 0.5
 
 
-@pytest.mark.parametrize("T", [29, 100, 224, 225, 300])
+@pytest.mark.parametrize("T", [29, 100, 224, 225, 300, 700])
 def test_wave_scales_far_apart_and_sequence_lengths(ops, T):
     """k jumps by +-60 between token ranges (every wave gets its own reference exponent, rescaled exactly
-    when aggregates cross waves); T = 224 is the longest tiled case, 225 and 300 take the sequential kernel."""
+    when aggregates cross waves); T = 224 is the longest single-launch case, longer ones take the three-launch
+    path (2 and 4 super-chunks)."""
     from oracle import biwkv
     B, C = 2, 64
     rng = np.random.default_rng(T)
@@ -137,3 +138,27 @@ def test_wave_scales_far_apart_and_sequence_lengths(ops, T):
     # cancels to ~1e-6 of its terms: fp32 keeps 5e-4 of the tensor's rms there (both kernels), not 1e-4
     assert rel_err(gk, rk) <= 5e-4 and rel_err(gv, rv) <= 5e-4
     assert rel_err(gw, rw) <= 5e-4 and rel_err(gu, ru) <= 5e-4
+
+
+def test_long_sequence_tiled_equals_sequential(ops, monkeypatch):
+    """VRWKV-L at 384x384 (T = 576, three super-chunks): the three-launch tiled path against the sequential
+    kernel, the float64 closed form on a slice, and the sum identities."""
+    B, T, C = 4, 576, 256
+    g = torch.Generator().manual_seed(11)
+    k = torch.randn(B, T, C, generator=g).cuda()
+    v = torch.randn(B, T, C, generator=g).cuda()
+    gy = torch.randn(B, T, C, generator=g).cuda()
+    w = ((torch.rand(C, generator=g) * 8 - 5) / T).cuda()
+    u = (torch.rand(C, generator=g) - 0.5).cuda()
+    got = ops.bi_wkv_backward(w, u, k, v, gy)
+    monkeypatch.setenv("VRWKV_BIWKV_BWD_PATH", "serial")
+    ref = ops.bi_wkv_backward(w, u, k, v, gy)
+    torch.cuda.synchronize()
+    for a, b, name in zip(got, ref, ("gw", "gu", "gk", "gv")):
+        assert rel_err(a.cpu().numpy(), b.cpu().numpy()) <= 5e-4, name
+    from oracle import biwkv
+    sl = (slice(0, 1), slice(None), slice(64, 128))
+    f = lambda x: x.cpu().numpy()
+    _, _, rk, rv = biwkv.biwkv_grads_closed(f(w[64:128]), f(u[64:128]), f(k[sl]), f(v[sl]), f(gy[sl]))
+    assert rel_err(f(got[2][sl]), rk) <= 1e-4 and rel_err(f(got[3][sl]), rv) <= 1e-4
+    assert (got[3].sum(1) - gy.sum(1)).abs().max().item() <= 1e-4 * gy.abs().sum(1).max().item()

@@ -54,40 +54,83 @@ int validate(int B, int T, int C, int io_dtype) {
     return VRWKV_OK;
 }
 
+// How a call is laid out: L tokens per wave, S waves per workgroup, nSC super-chunks per sequence
+// (L = 0: the sequential kernel), and where the pieces of the workspace are (in floats).
+struct BwdPlan {
+    int L = 0, S = 0, nSC = 1;
+    size_t planes = 0, agg1 = 0, agg2 = 0, parts = 0, total = 0;
+};
+
+BwdPlan make_bwd_plan(int B, int T, int C) {
+    BwdPlan p;
+    static const int kL[] = {4, 8, 16, 28};
+    const char* path = getenv("VRWKV_BIWKV_BWD_PATH");       // "serial" forces the sequential kernel (testing)
+    const bool tiled = !(path && path[0] == 's') && (long long)T * C < (1LL << 29);
+    if (tiled) {
+        for (int i = 3; i >= 0; --i)
+            if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX) p.L = kL[i];     // smallest L that fits: most waves per tile
+        if (p.L) {
+            p.S = (T + p.L - 1) / p.L;
+        } else {
+            p.L = 28; p.S = BWD_SMAX;
+            p.nSC = (T + p.S * p.L - 1) / (p.S * p.L);
+        }
+    }
+    p.planes = (size_t)5 * B * T * C;                        // sequential form: 5 floats per element
+    p.agg1 = (size_t)B * p.nSC * 5 * C;
+    p.agg2 = (size_t)B * p.nSC * BWD_SMAX * 9 * C;
+    p.parts = (size_t)2 * B * p.nSC * C;
+    p.total = p.planes + p.agg1 + p.agg2 + p.parts;
+    return p;
+}
+
+template <typename IO, int L>
+void launch_tiled(const BwdPlan& p, const float* w, const float* u, const IO* k, const IO* v, const IO* gy, IO* gk, IO* gv,
+                  float* ws, float* agg1, float* agg2, float* gw_part, float* gu_part, int B, int T, int C, hipStream_t st) {
+    BwdGeom geo;
+    geo.n_ctile = (C + WAVE - 1) / WAVE;
+    geo.nSC = p.nSC;
+    geo.n_tiles = B * p.nSC * geo.n_ctile;
+    const int per_cu = BWD_SMAX / p.S > 0 ? BWD_SMAX / p.S : 1;
+    int grid = biwkv_fwd_detail::num_cus() * per_cu;
+    if (grid > geo.n_tiles) grid = geo.n_tiles;
+    const dim3 g(grid), blk(p.S * WAVE);
+    if (p.nSC == 1) {
+        hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 0>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
+                           gw_part, gu_part, B, T, C, geo);
+    } else if constexpr (L == 28) {
+        hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 1>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
+                           gw_part, gu_part, B, T, C, geo);
+        hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 2>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
+                           gw_part, gu_part, B, T, C, geo);
+        hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 3>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
+                           gw_part, gu_part, B, T, C, geo);
+    }
+}
+
 template <typename IO>
 int launch(const float* w, const float* u, const void* k, const void* v, const void* gy, float* gw, float* gu,
            void* gk, void* gv, float* ws, int B, int T, int C, hipStream_t st) {
-    const size_t plane = (size_t)B * T * C;
-    float* gw_part = ws + 5 * plane;
-    float* gu_part = gw_part + (size_t)B * C;
+    const BwdPlan p = make_bwd_plan(B, T, C);
+    float* agg1 = ws + p.planes;
+    float* agg2 = agg1 + p.agg1;
+    float* gw_part = agg2 + p.agg2;
+    float* gu_part = gw_part + p.parts / 2;
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
     const IO* gg = static_cast<const IO*>(gy);
     IO* ok = static_cast<IO*>(gk);
     IO* ov = static_cast<IO*>(gv);
-    // sequences that fit one workgroup (8 waves x L tokens) take the tiled kernel
-    static const int kL[] = {4, 8, 16, 28};
-    int L = 0;
-    const char* path = getenv("VRWKV_BIWKV_BWD_PATH");       // "serial" forces the sequential kernel (testing)
-    if (!(path && path[0] == 's'))
-        for (int i = 3; i >= 0; --i)
-            if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX) L = kL[i];   // smallest L that fits: most waves per tile
-    if (L) {
-        const int S = (T + L - 1) / L;
-        const int n_ctile = (C + WAVE - 1) / WAVE;
-        const int n_tiles = B * n_ctile;
-        const int per_cu = BWD_SMAX / S > 0 ? BWD_SMAX / S : 1;
-        int grid = biwkv_fwd_detail::num_cus() * per_cu;
-        if (grid > n_tiles) grid = n_tiles;
-#define VRWKV_BWD_CASE(LL) case LL: hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, LL>), dim3(grid), dim3(S * WAVE), 0, st, \
-                           w, u, kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C, n_ctile, n_tiles); break;
-        switch (L) { VRWKV_BWD_CASE(4) VRWKV_BWD_CASE(8) VRWKV_BWD_CASE(16) VRWKV_BWD_CASE(28) }
-#undef VRWKV_BWD_CASE
-    } else {
-        hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
-                           kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C);
+    switch (p.L) {
+        case 4:  launch_tiled<IO, 4>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
+        case 8:  launch_tiled<IO, 8>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
+        case 16: launch_tiled<IO, 16>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
+        case 28: launch_tiled<IO, 28>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
+        default:
+            hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
+                               kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C);
     }
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gw_part, gw, gu_part, gu, B, C);
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gw_part, gw, gu_part, gu, B * p.nSC, C);
     return check_launch("biwkv_bwd");
 }
 
@@ -98,7 +141,7 @@ using namespace vrwkv;
 
 extern "C" size_t vrwkv_biwkv_bwd_workspace_bytes(int B, int T, int C, int io_dtype) {
     if (validate(B, T, C, io_dtype) != VRWKV_OK) return 0;
-    return ((size_t)5 * B * T * C + (size_t)2 * B * C) * sizeof(float);
+    return make_bwd_plan(B, T, C).total * sizeof(float);
 }
 
 extern "C" int vrwkv_biwkv_bwd(const float* w, const float* u, const void* k, const void* v, const void* gy,
@@ -110,7 +153,7 @@ extern "C" int vrwkv_biwkv_bwd(const float* w, const float* u, const void* k, co
         set_error("biwkv_bwd: null pointer argument");
         return VRWKV_INVALID_ARG;
     }
-    const size_t need = ((size_t)5 * B * T * C + (size_t)2 * B * C) * sizeof(float);
+    const size_t need = make_bwd_plan(B, T, C).total * sizeof(float);
     if (!workspace || workspace_bytes < need) {
         set_error("biwkv_bwd: workspace of %zu bytes required (got %zu)", need, workspace ? workspace_bytes : (size_t)0);
         return VRWKV_WORKSPACE_TOO_SMALL;

@@ -33,7 +33,8 @@ __device__ __forceinline__
 void biwkv_bwd_serial_seq(const float* __restrict__ w_, const float* __restrict__ u_,
                           const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
                           IO* __restrict__ gk_, IO* __restrict__ gv_, float* __restrict__ ws,
-                          float* __restrict__ gw_part, float* __restrict__ gu_part, int B, int T, int C, int b, int c)
+                          float* __restrict__ gw_part, float* __restrict__ gu_part, int B, int T, int C, int b, int c,
+                          int rows_per_batch = 1)
 {
     const float om = w_[c] * LOG2E, mu = u_[c] * LOG2E;
     const size_t base = (size_t)b * T * C + c;
@@ -103,8 +104,14 @@ void biwkv_bwd_serial_seq(const float* __restrict__ w_, const float* __restrict_
             g.push(om, z, z * y, -m);
         }
     }
-    gw_part[(size_t)b * C + c] = gw_acc;
-    gu_part[(size_t)b * C + c] = gu_acc;
+    // the partial-sum table has rows_per_batch rows per batch element (the tiled kernel writes one per
+    // super-chunk); the whole-sequence sums go to the first, zeros to the others
+    gw_part[(size_t)b * rows_per_batch * C + c] = gw_acc;
+    gu_part[(size_t)b * rows_per_batch * C + c] = gu_acc;
+    for (int r = 1; r < rows_per_batch; ++r) {
+        gw_part[((size_t)b * rows_per_batch + r) * C + c] = 0.f;
+        gu_part[((size_t)b * rows_per_batch + r) * C + c] = 0.f;
+    }
 }
 
 }  // namespace biwkv_bwd_detail

@@ -1,8 +1,14 @@
-// Bi-WKV backward, tiled kernel for sequences that fit one workgroup (T <= 8 waves x 28 tokens).
+// Bi-WKV backward, tiled kernel.
 //
 // Same decomposition as the forward kernel: lane = channel, wave = L consecutive tokens in registers,
-// workgroup = one (batch, 64 channels) tile, persistent workgroups walking the tiles.  k, v, gy are
-// read from HBM once and gk, gv written once; nothing else touches HBM except 2 floats per (b, c).
+// workgroup = S <= 8 waves = one (batch, super-chunk of S*L tokens, 64 channels) tile, persistent
+// workgroups walking the tiles.  When the sequence fits one super-chunk (T <= 224) k, v, gy are read
+// from HBM once and gk, gv written once (MODE 0).  Longer sequences take three launches, because both
+// scans need every other super-chunk's sums before they can finish:
+//   MODE 1  forward aggregates of every super-chunk                      (reads k, v)
+//   MODE 2  forward with carries -> z, z*y -> per-wave sums of the adjoint scans   (reads k, v, gy)
+//   MODE 3  the same again, then the adjoint scans with carries -> gk, gv          (reads k, v, gy)
+// i.e. 10 tensor passes instead of 5, through a small auxiliary table.
 //
 // With E_i = e^{k_i}, g = e^{-w}, cu = e^{u}:
 //   phase 1 (the forward):  D_t = sum_{i<t} g^{t-i-1} E_i + sum_{i>t} g^{i-t-1} E_i + cu E_t, N_t likewise
@@ -69,13 +75,21 @@ struct ZScan {
     }
 };
 
-template <typename IO, int L>
+// Auxiliary table of the long-sequence path (floats):
+//   agg1 [B][nSC][5][C]      forward aggregates of a super-chunk at its own scale R: A, B, R, Cg, D
+//   agg2 [B][nSC][8][9][C]   per wave: past-side sums (s0, s1, l0, l1), future-side sums, scale Re
+struct BwdGeom {
+    int n_ctile, nSC, n_tiles;      // tile id = (b * nSC + sc) * n_ctile + ctile
+};
+
+template <typename IO, int L, int MODE>
 __global__ __launch_bounds__(BWD_SMAX * WAVE)
 void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
                            const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
                            IO* __restrict__ gk_, IO* __restrict__ gv_,
-                           float* __restrict__ ws, float* __restrict__ gw_part, float* __restrict__ gu_part,
-                           int B, int T, int C, int n_ctile, int n_tiles)
+                           float* __restrict__ ws, float* __restrict__ agg1, float* __restrict__ agg2,
+                           float* __restrict__ gw_part, float* __restrict__ gu_part,
+                           int B, int T, int C, BwdGeom geo)
 {
     using Raw = typename BufRaw<sizeof(IO)>::type;
     __shared__ float s1[BWD_SMAX][5][WAVE];
@@ -85,21 +99,28 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int S = blockDim.x >> 6;
+    const int nSC = geo.nSC, n_ctile = geo.n_ctile, n_tiles = geo.n_tiles;
     const float NEG_INF = -__builtin_inff();
     const unsigned row = (unsigned)(C * sizeof(IO));
     const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
     auto shift_of = [](float d) -> int { return (int)fminf(fmaxf(d, -300.f), 300.f); };
 
     for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const int ctile = tile % n_ctile, b = tile / n_ctile;
+        const int ctile = tile % n_ctile;
+        const int sc = (tile / n_ctile) % nSC, b = tile / n_ctile / nSC;
         const int c0 = ctile * WAVE + lane;
         const bool cok = c0 < C;
-        const int tw = wave * L;
+        const int tw = (sc * S + wave) * L;
         const unsigned voff0 = cok ? (unsigned)(((size_t)tw * C + c0) * sizeof(IO)) : OOB_OFFSET;
         const size_t slab = (size_t)b * T * C;
         const float om = (cok ? w_[c0] : 0.f) * LOG2E;
         const float mu = (cok ? u_[c0] : 0.f) * LOG2E;
         if (!bwd_tile_is_fast(om, mu, T)) continue;          // workgroup-uniform: same channels in every wave
+        const int cc = cok ? c0 : 0;                         // in-range column for the auxiliary table
+        auto a1 = [&](int s, int slot) -> float& { return agg1[(((size_t)b * nSC + s) * 5 + slot) * C + cc]; };
+        auto a2 = [&](int s, int wv, int slot) -> float& {
+            return agg2[((((size_t)b * nSC + s) * BWD_SMAX + wv) * 9 + slot) * C + cc];
+        };
 
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes);
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
@@ -111,9 +132,11 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             Kr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rk, vo, 0);
             Vr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rv, vo, 0);
         }
+        if (MODE != 1) {
 #pragma unroll
-        for (int j = 0; j < L; ++j)
-            Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
+            for (int j = 0; j < L; ++j)
+                Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
+        }
 
         const float gd = fast_exp2(-om), cu = fast_exp2(mu);
         const float G = fast_exp2(-om * (float)L);
@@ -159,9 +182,48 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                 lc[s] = s1[ss][3][lane]; ld[s] = s1[ss][4][lane];
             }
             float r = NEG_BIG;
+            if (MODE >= 2) {
+                for (int s = 0; s < nSC; ++s) r = fmaxf(r, a1(s, 2));       // common scale of the whole sequence
+            } else {
 #pragma unroll
-            for (int s = 0; s < BWD_SMAX; ++s) r = fmaxf(r, lr[s]);
+                for (int s = 0; s < BWD_SMAX; ++s) r = fmaxf(r, lr[s]);
+            }
             r = (r > NEG_BIG) ? r : 0.f;
+            if (MODE == 1) {
+                // fold the waves into the super-chunk's aggregates (both referenced to its ends) and publish
+#pragma unroll
+                for (int s = 0; s < BWD_SMAX; ++s)
+                    if (s < S) {
+                        const int sh = shift_of(lr[s] - r);
+                        a = fmaf(G, a, ldexpf(la[s], sh));
+                        bb = fmaf(G, bb, ldexpf(lb[s], sh));
+                    }
+#pragma unroll
+                for (int s = BWD_SMAX - 1; s >= 0; --s)
+                    if (s < S) {
+                        const int sh = shift_of(lr[s] - r);
+                        c = fmaf(G, c, ldexpf(lc[s], sh));
+                        d = fmaf(G, d, ldexpf(ld[s], sh));
+                    }
+                if (wave == 0 && cok) {
+                    a1(sc, 0) = a; a1(sc, 1) = bb; a1(sc, 2) = r; a1(sc, 3) = c; a1(sc, 4) = d;
+                }
+                lds_barrier();                                // s1 is rewritten by the next tile
+                continue;
+            }
+            if (MODE >= 2) {
+                const float GS = fast_exp2(-om * (float)(S * L));
+                for (int s = 0; s < sc; ++s) {
+                    const int sh = shift_of(a1(s, 2) - r);
+                    a = fmaf(GS, a, ldexpf(a1(s, 0), sh));
+                    bb = fmaf(GS, bb, ldexpf(a1(s, 1), sh));
+                }
+                for (int s = nSC - 1; s > sc; --s) {
+                    const int sh = shift_of(a1(s, 2) - r);
+                    c = fmaf(GS, c, ldexpf(a1(s, 3), sh));
+                    d = fmaf(GS, d, ldexpf(a1(s, 4), sh));
+                }
+            }
 #pragma unroll
             for (int s = 0; s < BWD_SMAX; ++s)
                 if (s < wave) {
@@ -211,6 +273,16 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
 #pragma unroll
         for (int j = 0; j < L; ++j) pl.push(gd, Z[j], ZY[j]);
 
+        if (MODE == 2) {
+            if (cok) {
+                a2(sc, wave, 0) = pl.s0; a2(sc, wave, 1) = pl.s1; a2(sc, wave, 2) = pl.l0; a2(sc, wave, 3) = pl.l1;
+                a2(sc, wave, 4) = fl.s0; a2(sc, wave, 5) = fl.s1; a2(sc, wave, 6) = fl.l0; a2(sc, wave, 7) = fl.l1;
+                a2(sc, wave, 8) = Re;
+            }
+            lds_barrier();                                    // s1 is rewritten by the next tile
+            continue;
+        }
+
         // ------------------------------ phase 2: the adjoint ------------------------------
         s2[wave][0][lane] = pl.s0; s2[wave][1][lane] = pl.s1; s2[wave][2][lane] = pl.l0; s2[wave][3][lane] = pl.l1;
         s2[wave][4][lane] = fl.s0; s2[wave][5][lane] = fl.s1; s2[wave][6][lane] = fl.l0; s2[wave][7][lane] = fl.l1;
@@ -220,6 +292,21 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         ZScan p, f;
         {
             const float nL = (float)L;
+            if (MODE == 3) {
+                // every wave of the other super-chunks, nearest last (they all span L token positions)
+                for (int s = 0; s < sc; ++s)
+                    for (int wv = 0; wv < BWD_SMAX; ++wv) {
+                        const int sh = shift_of(Rw - a2(s, wv, 8));
+                        p.hop(G, nL, ldexpf(a2(s, wv, 0), sh), ldexpf(a2(s, wv, 1), sh),
+                              ldexpf(a2(s, wv, 2), sh), ldexpf(a2(s, wv, 3), sh));
+                    }
+                for (int s = nSC - 1; s > sc; --s)
+                    for (int wv = BWD_SMAX - 1; wv >= 0; --wv) {
+                        const int sh = shift_of(Rw - a2(s, wv, 8));
+                        f.hop(G, nL, ldexpf(a2(s, wv, 4), sh), ldexpf(a2(s, wv, 5), sh),
+                              ldexpf(a2(s, wv, 6), sh), ldexpf(a2(s, wv, 7), sh));
+                    }
+            }
 #pragma unroll
             for (int s = 0; s < BWD_SMAX; ++s)
                 if (s < wave) {
@@ -256,27 +343,29 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             store1<IO>(rgk, vo, gk);
         }
 
-        // per-(b, c) partial sums of gw, gu: over this wave's tokens, then over the waves
+        // partial sums of gw, gu per (b, super-chunk, c): over this wave's tokens, then over the waves
         s3[wave][0][lane] = gw_acc;
         s3[wave][1][lane] = gu_acc;
         lds_barrier();
         if (wave == 0 && cok) {
             float sw = 0.f, su = 0.f;
             for (int s = 0; s < S; ++s) { sw += s3[s][0][lane]; su += s3[s][1][lane]; }
-            gw_part[(size_t)b * C + c0] = sw;
-            gu_part[(size_t)b * C + c0] = su;
+            gw_part[((size_t)b * nSC + sc) * C + c0] = sw;
+            gu_part[((size_t)b * nSC + sc) * C + c0] = su;
         }
     }
 
-    // second walk: tiles outside the plain-sum regime, one wave per tile, sequential form
-    for (int tile = blockIdx.x * S + wave; tile < n_tiles; tile += gridDim.x * S) {
-        const int ctile = tile % n_ctile, b = tile / n_ctile;
+    if (MODE == 1 || MODE == 2) return;
+    // second walk: (batch, channel tile) pairs outside the plain-sum regime, one wave each, sequential form
+    const int n_pairs = n_tiles / nSC;
+    for (int pair = blockIdx.x * S + wave; pair < n_pairs; pair += gridDim.x * S) {
+        const int ctile = pair % n_ctile, b = pair / n_ctile;
         const int c0 = ctile * WAVE + lane;
         const bool cok = c0 < C;
         const float om = (cok ? w_[c0] : 0.f) * LOG2E;
         const float mu = (cok ? u_[c0] : 0.f) * LOG2E;
         if (bwd_tile_is_fast(om, mu, T)) continue;
-        if (cok) biwkv_bwd_serial_seq<IO>(w_, u_, k_, v_, gy_, gk_, gv_, ws, gw_part, gu_part, B, T, C, b, c0);
+        if (cok) biwkv_bwd_serial_seq<IO>(w_, u_, k_, v_, gy_, gk_, gv_, ws, gw_part, gu_part, B, T, C, b, c0, nSC);
     }
 }
 
