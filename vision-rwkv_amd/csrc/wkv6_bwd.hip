@@ -23,7 +23,9 @@
 //   sweep S (ascending)   own = key j:    S  -> gr, a (workspace), gu partial
 //   sweep G (descending)  own = key j:    G  -> gk, gw
 //   sweep V (descending)  own = value i:  G^T -> gv
-#include "vrwkv_common.h"
+#include "wkv6_bwd_chunk.h"
+#include <cstdlib>
+#include <type_traits>
 
 namespace vrwkv {
 namespace {
@@ -48,8 +50,8 @@ __device__ __forceinline__ float log_decay(const WT* w_, size_t o) {
 
 // ---- sweep S: state S, own = j ----------------------------------------------------------------
 template <typename IO, typename WT, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(256)
-void wkv6_bwd_sweep_s(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
+__device__ __forceinline__
+void wkv6_bwd_sweep_s_body(int bh, const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
                       const WT* __restrict__ w_, const float* __restrict__ u_, const float* __restrict__ gy_,
                       float* __restrict__ gr_, float* __restrict__ a_, float* __restrict__ gu_part,
                       int T, int C, int H)
@@ -57,7 +59,7 @@ void wkv6_bwd_sweep_s(const IO* __restrict__ r_, const IO* __restrict__ k_, cons
     __shared__ __attribute__((aligned(16))) float s_row[4][2][N];       // [wave][v, gy][i]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int b = bh / H, h = bh % H;
     const int sq = lane & 3, j = wave * 16 + (lane >> 2);
     const size_t base = (size_t)b * T * C + (size_t)h * N;
     const float uj = DIR == 0 ? u_[h * N + j] : 0.f;
@@ -101,8 +103,8 @@ void wkv6_bwd_sweep_s(const IO* __restrict__ r_, const IO* __restrict__ k_, cons
 
 // ---- sweep G: adjoint G, own = j, descending in pass order ---------------------------------------
 template <typename IO, typename WT, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(256)
-void wkv6_bwd_sweep_g(const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
+__device__ __forceinline__
+void wkv6_bwd_sweep_g_body(int bh, const IO* __restrict__ r_, const IO* __restrict__ k_, const IO* __restrict__ v_,
                       const WT* __restrict__ w_, const float* __restrict__ u_, const float* __restrict__ gy_,
                       const float* __restrict__ a_, float* __restrict__ gk_, float* __restrict__ gw_,
                       int T, int C, int H)
@@ -110,7 +112,7 @@ void wkv6_bwd_sweep_g(const IO* __restrict__ r_, const IO* __restrict__ k_, cons
     __shared__ __attribute__((aligned(16))) float s_row[4][2][N];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int b = bh / H, h = bh % H;
     const int sq = lane & 3, j = wave * 16 + (lane >> 2);
     const size_t base = (size_t)b * T * C + (size_t)h * N;
     const float uj = DIR == 0 ? u_[h * N + j] : 0.f;
@@ -155,15 +157,15 @@ void wkv6_bwd_sweep_g(const IO* __restrict__ r_, const IO* __restrict__ k_, cons
 
 // ---- sweep V: adjoint G^T, own = i, descending in pass order --------------------------------------
 template <typename IO, typename WT, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(256)
-void wkv6_bwd_sweep_v(const IO* __restrict__ r_, const IO* __restrict__ k_,
+__device__ __forceinline__
+void wkv6_bwd_sweep_v_body(int bh, const IO* __restrict__ r_, const IO* __restrict__ k_,
                       const WT* __restrict__ w_, const float* __restrict__ u_, const float* __restrict__ gy_,
                       float* __restrict__ gv_, int T, int C, int H)
 {
     __shared__ __attribute__((aligned(16))) float s_row[4][3][N];       // [wave][r, k, d][j]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int b = bh / H, h = bh % H;
     const int sq = lane & 3, i = wave * 16 + (lane >> 2);
     const size_t base = (size_t)b * T * C + (size_t)h * N;
     float uu[16];
@@ -203,6 +205,43 @@ void wkv6_bwd_sweep_v(const IO* __restrict__ r_, const IO* __restrict__ k_,
     }
 }
 
+// ---- kernels: one sweep each (sequential path), or all six for the sequences the chunked scans left ----
+template <typename IO, typename WT, int DIR, bool W_IS_EW>
+__global__ __launch_bounds__(256)
+void wkv6_bwd_sweep_s(const IO* r_, const IO* k_, const IO* v_, const WT* w_, const float* u_, const float* gy_,
+                      float* gr_, float* a_, float* gu_part, int T, int C, int H) {
+    wkv6_bwd_sweep_s_body<IO, WT, DIR, W_IS_EW>(blockIdx.x, r_, k_, v_, w_, u_, gy_, gr_, a_, gu_part, T, C, H);
+}
+template <typename IO, typename WT, int DIR, bool W_IS_EW>
+__global__ __launch_bounds__(256)
+void wkv6_bwd_sweep_g(const IO* r_, const IO* k_, const IO* v_, const WT* w_, const float* u_, const float* gy_,
+                      const float* a_, float* gk_, float* gw_, int T, int C, int H) {
+    wkv6_bwd_sweep_g_body<IO, WT, DIR, W_IS_EW>(blockIdx.x, r_, k_, v_, w_, u_, gy_, a_, gk_, gw_, T, C, H);
+}
+template <typename IO, typename WT, int DIR, bool W_IS_EW>
+__global__ __launch_bounds__(256)
+void wkv6_bwd_sweep_v(const IO* r_, const IO* k_, const WT* w_, const float* u_, const float* gy_,
+                      float* gv_, int T, int C, int H) {
+    wkv6_bwd_sweep_v_body<IO, WT, DIR, W_IS_EW>(blockIdx.x, r_, k_, w_, u_, gy_, gv_, T, C, H);
+}
+// Sequences flagged by the chunked scans (a chunk decaying below e^-60): all six sweeps, descending pass
+// first.  Every sweep maps (token, channel) to the same thread as the sweep it depends on, so program
+// order is enough between them.
+template <typename IO, typename WT, bool W_IS_EW>
+__global__ __launch_bounds__(256)
+void wkv6_bwd_fallback(const IO* r_, const IO* k_, const IO* v_, const WT* w_, const float* u_, const float* gy_,
+                       float* gr_, float* gk_, float* gv_, float* gw_, float* a_, float* gu_part,
+                       const unsigned char* todo, int T, int C, int H) {
+    const int bh = blockIdx.x;
+    if (!todo[bh]) return;
+    wkv6_bwd_sweep_s_body<IO, WT, 1, W_IS_EW>(bh, r_, k_, v_, w_, u_, gy_, gr_, a_, gu_part, T, C, H);
+    wkv6_bwd_sweep_g_body<IO, WT, 1, W_IS_EW>(bh, r_, k_, v_, w_, u_, gy_, a_, gk_, gw_, T, C, H);
+    wkv6_bwd_sweep_v_body<IO, WT, 1, W_IS_EW>(bh, r_, k_, w_, u_, gy_, gv_, T, C, H);
+    wkv6_bwd_sweep_s_body<IO, WT, 0, W_IS_EW>(bh, r_, k_, v_, w_, u_, gy_, gr_, a_, gu_part, T, C, H);
+    wkv6_bwd_sweep_g_body<IO, WT, 0, W_IS_EW>(bh, r_, k_, v_, w_, u_, gy_, a_, gk_, gw_, T, C, H);
+    wkv6_bwd_sweep_v_body<IO, WT, 0, W_IS_EW>(bh, r_, k_, w_, u_, gy_, gv_, T, C, H);
+}
+
 template <typename IO, typename WT, bool EW>
 int launch_all(const void* r, const void* k, const void* v, const void* w, const float* u, const float* gy,
                float* gr, float* gk, float* gv, float* gw, float* gu, float* ws, int B, int T, int C, int H, hipStream_t st) {
@@ -213,6 +252,24 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
     float* a = ws;                                       // (B,T,C)
     float* gu_part = ws + (size_t)B * T * C;             // (B,C)
     const dim3 grid(B * H), block(256);
+    if constexpr (std::is_same<IO, __hip_bfloat16>::value) {
+        const char* path = getenv("VRWKV_WKV6_BWD_PATH");            // "scalar" forces the sequential sweeps (testing)
+        if (!(path && path[0] == 's') && (long long)T * C < (1LL << 29)) {
+            using namespace wkv6_detail;
+            unsigned char* todo = reinterpret_cast<unsigned char*>(gu_part + (size_t)B * C);
+            const dim3 blk(128);
+#define VRWKV_SCAN(KIND, DIR, OUT) hipLaunchKernelGGL((wkv6_bwd_scan_kernel<WT, KIND, DIR, EW>), grid, blk, 0, st, \
+                                                      rr, kk, vv, ww, u, gy, OUT, a, gw, gu_part, todo, T, C, H)
+            VRWKV_SCAN(SCAN_GR, 1, gr); VRWKV_SCAN(SCAN_GK, 1, gk); VRWKV_SCAN(SCAN_GV, 1, gv);
+            VRWKV_SCAN(SCAN_GR, 0, gr); VRWKV_SCAN(SCAN_GK, 0, gk); VRWKV_SCAN(SCAN_GV, 0, gv);
+#undef VRWKV_SCAN
+            hipLaunchKernelGGL((wkv6_bwd_fallback<IO, WT, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, gr, gk, gv, gw,
+                               a, gu_part, todo, T, C, H);
+            hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gu_part, gu, (const float*)nullptr,
+                               (float*)nullptr, B, C);
+            return check_launch("wkv6_bwd (chunked)");
+        }
+    }
     // descending pass first (writes), ascending pass second (accumulates), as in the forward
     hipLaunchKernelGGL((wkv6_bwd_sweep_s<IO, WT, 1, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, gr, a, gu_part, T, C, H);
     hipLaunchKernelGGL((wkv6_bwd_sweep_g<IO, WT, 1, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, a, gk, gw, T, C, H);
@@ -231,7 +288,7 @@ using namespace vrwkv;
 
 extern "C" size_t vrwkv_wkv6_bwd_workspace_bytes(int B, int T, int C, int H) {
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return 0;
-    return ((size_t)B * T * C + (size_t)B * C) * sizeof(float);
+    return ((size_t)B * T * C + (size_t)B * C) * sizeof(float) + (((size_t)B * H + 255) & ~(size_t)255);
 }
 
 extern "C" int vrwkv_wkv6_bwd(const void* r, const void* k, const void* v, const void* w, const float* u,
@@ -259,7 +316,7 @@ extern "C" int vrwkv_wkv6_bwd(const void* r, const void* k, const void* v, const
         set_error("wkv6_bwd: null pointer argument");
         return VRWKV_INVALID_ARG;
     }
-    const size_t need = ((size_t)B * T * C + (size_t)B * C) * sizeof(float);
+    const size_t need = ((size_t)B * T * C + (size_t)B * C) * sizeof(float) + (((size_t)B * H + 255) & ~(size_t)255);
     if (!workspace || workspace_bytes < need) {
         set_error("wkv6_bwd: workspace of %zu bytes required (got %zu)", need, workspace ? workspace_bytes : (size_t)0);
         return VRWKV_WORKSPACE_TOO_SMALL;

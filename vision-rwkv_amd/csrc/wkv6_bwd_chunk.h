@@ -1,0 +1,416 @@
+// wkv6 backward, chunked matrix-core scans for gfx950 (bf16 MFMA, fp32 accumulate; bf16 r, k, v).
+//
+// One causal pass of the forward (tokens in pass order n, state S_n before token n, d_n = exp(ld_n)):
+//   y_n = r_n (diag(u) k_n v_n^T + S_n),   S_{n+1} = diag(d_n) S_n + k_n v_n^T
+// and its adjoint state G_n = r_n gy_n^T + diag(d_n) G_{n+1} give
+//   gr_n[j] = u_j k_n[j] (v_n.gy_n) + (S_n gy_n)[j]            scan GR  (pass order,     state S^T[i][j])
+//   gk_n[j] = u_j r_n[j] (v_n.gy_n) + (G_{n+1} v_n)[j]         scan GK  (reverse order,  state G^T[i][j])
+//   gv_n[i] = sum_j k_n[j] (u_j r_n[j] gy_n[i] + G_{n+1}[j,i]) scan GV  (reverse order,  state G[j][i])
+//   gw_n[j] = ld_n[j] ( sum_{m>n} (a_m - b_m) - b_n ),  a = r (S gy),  b = k (G v)   (GR stores a, GK finishes gw)
+// (formulas of classification/mmcls_custom/models/backbones/cuda_v6/wkv6_cuda.cu:99-346).
+//
+// Every scan is the same chunked algorithm as the forward kernel, on 32-token chunks, with other operands.
+// In scan order rho (the pass order or its reverse) and with c the contracted channel, o the output channel:
+//   A[t][s]   = sum_c Q[t][c] Kc[s][c]   (s before t in scan order; the bonus on the diagonal for GV)
+//   Out[t][o] = sum_s A[t][s] Val[s][o]  +  sum_c Q[t][c] (state, rescaled)[c][o]
+//   state'    = decay * state + scale * sum_s Kc[s][c] Val[s][o]
+// With P the in-chunk cumulative log decay in PASS order, Pex = P - ld, Pref = P_15, f1 = e^(Pex-Pref),
+// f2 = e^(Pref-P), rt = r f1, kt = k f2, c1 = e^Pref, c2 = e^P31, c3 = e^(P31-Pref):
+//   GR: Q = gy, Kc = v,  Val = kt, state read * c1[j], update c2[j], c3[j];  gr = f1 Out + u k A[t][t], a = r f1 Out
+//   GK: Q = v,  Kc = gy, Val = rt, state read * c3[j], update c2[j], c1[j];  gk = f2 Out + u r A[t][t], b = k f2 Out
+//   GV: Q = kt, Kc = rt, Val = gy, state read * c3[j] (rows), update c2[j], c1[j] (rows);  gv = Out
+// GR and GK contract over the value channel i and own output columns j (the state is kept transposed, so its
+// decay is a per-lane factor); GV contracts over j like the forward.  The state never leaves the accumulator
+// registers; computed operands are split into bf16 head + tail (hh + ht + th), loaded bf16 ones are exact.
+//
+// One 128-thread workgroup per (b,h) and pass; the descending pass is launched first and writes, the
+// ascending pass adds (old values fetched behind the matrix stage).  A sequence with a chunk that decays by
+// more than e^-60 is flagged in `todo` and left to the sequential kernels.
+#pragma once
+#include "wkv6_fwd_chunk.h"
+
+namespace vrwkv {
+namespace wkv6_detail {
+
+enum { SCAN_GR = 0, SCAN_GK = 1, SCAN_GV = 2 };
+
+template <bool QS, bool KS>
+struct __attribute__((aligned(16))) ScanLds {
+    __bf16 Qh[LC][PJ], Ql[QS ? LC : 1][PJ];               // Q rows   [rho][c]
+    __bf16 Kh[LC][PJ], Kl[KS ? LC : 1][PJ];               // Kc rows  [rho][c]
+    __bf16 KTh[HN][PS], KTl[KS ? HN : 1][PS];             // Kc^T     [c][rho]
+    __bf16 VTh[HN][PS], VTl[HN][PS];                      // Val^T    [o][rho]
+    float Post[LC][HN];                                   // f1 / f2 in [rho][j]  (GR, GK)
+    float C1[HN], C2[HN], C3[HN], Tot[HN], Bon[4][LC], Diag[LC];
+};
+
+// DIR 0: ascending pass (bonus u, adds to the outputs).  DIR 1: descending pass (writes them).
+template <typename WT, int KIND, int DIR, bool W_IS_EW>
+__global__ __launch_bounds__(128)
+void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfloat16* __restrict__ k_,
+                          const __hip_bfloat16* __restrict__ v_, const WT* __restrict__ w_,
+                          const float* __restrict__ u_, const float* __restrict__ gy_,
+                          float* __restrict__ out_,        // gr / gk / gv
+                          float* __restrict__ a_,          // GR: written; GK: read
+                          float* __restrict__ gw_,         // GK
+                          float* __restrict__ gu_part,     // GR, DIR 0
+                          unsigned char* __restrict__ todo, int T, int C, int H)
+{
+    using IO = __hip_bfloat16;
+    constexpr bool REV = KIND != SCAN_GR;                  // scan order = reverse pass order
+    constexpr bool TT = KIND != SCAN_GV;                   // transposed state: contraction over i, output columns j
+    constexpr bool QS = KIND != SCAN_GK;                   // Q is computed (gy, kt) -> split; v is exact
+    constexpr bool KS = KIND != SCAN_GR;                   // Kc is computed (gy, rt) -> split; v is exact
+    constexpr bool ASC = DIR == 0;
+    constexpr bool LL = KIND != SCAN_GV;                   // tail x tail products too: gw is a difference of these sums
+    __shared__ ScanLds<QS, KS> L;
+    __shared__ int sFlag;
+
+    const int lane = threadIdx.x & 63;
+    const int q = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 5, x = lane & 31;
+    const int bh = blockIdx.x;
+    const int b = bh / H, h = bh % H;
+    const size_t base = (size_t)b * T * C + (size_t)h * HN;
+    const int nchunk = (T + LC - 1) / LC;
+    const int ocol = 32 * q + x;                           // output column of this lane in the matrix stage
+    const float u_e = ASC ? u_[h * HN + lane] : 0.f;       // bonus weight of the elementwise stage's channel
+    const float u_o = ASC ? u_[h * HN + ocol] : 0.f;       // ... and of the output column (GR, GK)
+    if (threadIdx.x == 0) sFlag = 0;
+    __syncthreads();
+
+    using RawIO = typename BufRaw<2>::type;
+    using RawW = typename BufRaw<sizeof(WT)>::type;
+    const unsigned span_io = (unsigned)(((size_t)(T - 1) * C + HN) * 2);
+    const unsigned span_w = (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(WT));
+    const unsigned span_f = (unsigned)(((size_t)(T - 1) * C + HN) * 4);
+    const __amdgpu_buffer_rsrc_t rsr = make_rsrc(r_ + base, span_io), rsk = make_rsrc(k_ + base, span_io),
+                                 rsv = make_rsrc(v_ + base, span_io), rsw = make_rsrc(w_ + base, span_w),
+                                 rsg = make_rsrc(gy_ + base, span_f), rso = make_rsrc(out_ + base, span_f);
+    const __amdgpu_buffer_rsrc_t rsa = make_rsrc((KIND != SCAN_GV ? a_ : out_) + base, span_f);
+    const __amdgpu_buffer_rsrc_t rsgw = make_rsrc((KIND == SCAN_GK ? gw_ : out_) + base, span_f);
+    auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, 2); return to_f32(t); };
+    auto cvtw = [](RawW raw) { WT t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
+
+    // Chunks are 32-token blocks of the token axis.  The scan walks them upwards when (ascending pass) !=
+    // (reversed scan), downwards otherwise; pass index n inside a chunk is token 32c + n (ascending pass) or
+    // 32c + 31 - n (descending); scan row rho = n, or 31 - n for a reversed scan.
+    constexpr bool UP = ASC != REV;
+    auto chunk_of = [&](int ch) { return UP ? ch : nchunk - 1 - ch; };
+    auto token_of_n = [&](int c, int n) { return c * LC + (ASC ? n : LC - 1 - n); };
+    // matrix-stage register r of a lane <-> scan row rho = 8(r/4) + 4g + (r%4) <-> token 32c + (UP ? rho : 31-rho)
+    const unsigned o_lane = (unsigned)(((UP ? 4 * g : 4 * (1 - g)) * C + ocol) * 4);
+    auto row_off = [&](int c, int r, int C, int esz) -> unsigned {   // byte offset of (token of register r, column ocol)
+        const int rl = 8 * (r / 4) + (r % 4);
+        return (o_lane / 4) * esz + (unsigned)((c * LC + (UP ? rl : 27 - rl)) * C * esz);
+    };
+
+    f32x16 S0 = {0}, S1 = {0};      // state tiles: rows c = 32*ch2 + 8(r/4)+4g+(r%4), column o = ocol
+    float xcarry = 0.f, gu_acc = 0.f;   // GK: sum of (a - b) over the tokens scanned so far; GR: gu
+    RawW wraw[16];
+    auto fetch_w = [&](int ch, int C) {
+        const int c = chunk_of(ch);
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const int t = token_of_n(c, 16 * q + m);
+            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(WT));
+        }
+    };
+    fetch_w(0, C);
+
+    for (int ch = 0; ch < nchunk; ++ch) {
+        int Cs = C;
+        asm volatile("" : "+s"(Cs));                       // keep row offsets out of the loop-invariant scalars
+        const int cc = chunk_of(ch);
+        // =============================== stage E: elementwise =================================
+        // wave q prepares pass indices n = 16q .. 16q+15 of the chunk; lane = channel
+        RawIO xraw[16], yraw[16];                          // the two bf16 tensors this scan needs here
+        unsigned graw[16];                                 // gy (fp32 bits)
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const int t = token_of_n(cc, 16 * q + m);
+            const unsigned tt = (unsigned)(t < T ? t : 0);
+            const unsigned so = tt * Cs * 2u, vo = lane * 2u;
+            if (KIND == SCAN_GR) { xraw[m] = BufRaw<2>::ld(rsv, vo, so); yraw[m] = BufRaw<2>::ld(rsk, vo, so); }
+            if (KIND == SCAN_GK) { xraw[m] = BufRaw<2>::ld(rsv, vo, so); yraw[m] = BufRaw<2>::ld(rsr, vo, so); }
+            if (KIND == SCAN_GV) { xraw[m] = BufRaw<2>::ld(rsk, vo, so); yraw[m] = BufRaw<2>::ld(rsr, vo, so); }
+            graw[m] = BufRaw<4>::ld(rsg, lane * 4u, tt * Cs * 4u);
+        }
+        float ld[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const bool ok = token_of_n(cc, 16 * q + m) < T;
+            const float fw = cvtw(wraw[m]);
+            ld[m] = ok ? (W_IS_EW ? fw : -__expf(fw)) : 0.f;
+        }
+        float p[16];
+        p[0] = ld[0];
+#pragma unroll
+        for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
+        if (q == 0) L.Tot[lane] = p[15];
+        lds_barrier();                                                   // (1)
+        const float pref = L.Tot[lane];                                  // P_15
+        const float off = q == 1 ? pref : 0.f;
+        if (q == 1) {
+            const float p31 = p[15] + off;
+            L.C2[lane] = __expf(p31);
+            L.C3[lane] = __expf(p31 - pref);
+            if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY)) != 0ull && lane == 0) sFlag = 1;
+        } else {
+            L.C1[lane] = __expf(pref);
+        }
+        {
+            bf16x8 kth[2], ktl[2], vth[2], vtl[2];
+            float pu[16];
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                const int n = 16 * q + m;
+                const int rho = REV ? LC - 1 - n : n;
+                const int e = REV ? 15 - m : m;                           // position inside this wave's 16 rows
+                const bool ok = token_of_n(cc, n) < T;
+                const float P = p[m] + off;
+                const float f1 = __expf(P - ld[m] - pref);               // exp(Pex - Pref)
+                const float f2 = __expf(pref - P);                        // exp(Pref - P)
+                const float xa = ok ? cvt(xraw[m]) : 0.f, ya = ok ? cvt(yraw[m]) : 0.f;
+                const float gyv = ok ? __builtin_bit_cast(float, graw[m]) : 0.f;
+                // per scan: Q value, Kc value, Val value of this (token, channel)
+                float qv, kcv, valv;
+                if (KIND == SCAN_GR) { qv = gyv; kcv = xa; valv = ya * f2; L.Post[rho][lane] = f1; }
+                if (KIND == SCAN_GK) { qv = xa; kcv = gyv; valv = ya * f1; L.Post[rho][lane] = f2; }
+                if (KIND == SCAN_GV) { qv = xa * f2; kcv = ya * f1; valv = gyv; pu[m] = ya * u_e * xa; }
+                const __bf16 qh = (__bf16)qv, kh = (__bf16)kcv, vh = (__bf16)valv;
+                L.Qh[rho][lane] = qh;
+                if (QS) L.Ql[rho][lane] = (__bf16)(qv - (float)qh);
+                L.Kh[rho][lane] = kh;
+                kth[e >> 3][e & 7] = kh;
+                if (KS) {
+                    const __bf16 kl = (__bf16)(kcv - (float)kh);
+                    L.Kl[rho][lane] = kl;
+                    ktl[e >> 3][e & 7] = kl;
+                }
+                vth[e >> 3][e & 7] = vh;
+                vtl[e >> 3][e & 7] = (__bf16)(valv - (float)vh);
+            }
+            const int r0 = REV ? 16 * (1 - q) : 16 * q;                   // first scan row of this wave's block
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                *reinterpret_cast<bf16x8*>(&L.KTh[lane][r0 + 8 * e]) = kth[e];
+                if (KS) *reinterpret_cast<bf16x8*>(&L.KTl[lane][r0 + 8 * e]) = ktl[e];
+                *reinterpret_cast<bf16x8*>(&L.VTh[lane][r0 + 8 * e]) = vth[e];
+                *reinterpret_cast<bf16x8*>(&L.VTl[lane][r0 + 8 * e]) = vtl[e];
+            }
+            if (KIND == SCAN_GV && ASC) {                                 // bonus_n = sum_j r_n[j] u[j] k_n[j]
+                int idx;
+                const float rs = row_sums16(pu, lane, idx);
+                const int n = 16 * q + idx;
+                L.Bon[lane >> 4][REV ? LC - 1 - n : n] = rs;
+            }
+        }
+        lds_barrier();                                                   // (2)
+        if (sFlag) {                                                      // out of range: left to the sequential kernels
+            if (threadIdx.x == 0) todo[bh] = 1;
+            return;
+        }
+        if (ch + 1 < nchunk) fetch_w(ch + 1, Cs);                         // next chunk's decays, behind the matrix stage
+
+        // ================================= stage M: matrix cores ===============================
+        // values the epilogue needs in the output layout (lane = column ocol, register r = scan row)
+        float prev[16];
+        RawIO rraw[16], kraw[16];
+        unsigned araw[16], pgw[16];
+        RawW wo[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
+            if (KIND != SCAN_GV) {
+                rraw[r] = BufRaw<2>::ld(rsr, row_off(cc, r, Cs, 2), 0);
+                kraw[r] = BufRaw<2>::ld(rsk, row_off(cc, r, Cs, 2), 0);
+            }
+            if (KIND == SCAN_GK) {
+                araw[r] = BufRaw<4>::ld(rsa, row_off(cc, r, Cs, 4), 0);
+                wo[r] = BufRaw<sizeof(WT)>::ld(rsw, row_off(cc, r, Cs, sizeof(WT)), 0);
+                pgw[r] = ASC ? BufRaw<4>::ld(rsgw, row_off(cc, r, Cs, 4), 0) : 0u;
+            }
+        }
+        // ---- MFMA 1: A^T: acc[s][t] = sum_c Kc[s][c] Q[t][c]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
+        f32x16 accA = {0};
+#pragma unroll
+        for (int kq = 0; kq < 4; ++kq) {
+            const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&L.Kh[x][16 * kq + 8 * g]);
+            const bf16x8 bh_ = *reinterpret_cast<const bf16x8*>(&L.Qh[x][16 * kq + 8 * g]);
+            accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh_, accA, 0, 0, 0);
+            if (QS) {
+                const bf16x8 bl = *reinterpret_cast<const bf16x8*>(&L.Ql[x][16 * kq + 8 * g]);
+                accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, accA, 0, 0, 0);
+            }
+            if (KS) {
+                const bf16x8 al = *reinterpret_cast<const bf16x8*>(&L.Kl[x][16 * kq + 8 * g]);
+                accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh_, accA, 0, 0, 0);
+            }
+        }
+        const float bon = (KIND == SCAN_GV && ASC) ? (L.Bon[0][x] + L.Bon[1][x]) + (L.Bon[2][x] + L.Bon[3][x]) : 0.f;
+        bf16x8 Ah[2], Al[2];
+        int dx = 4 * g - x;
+        asm volatile("" : "+v"(dx));
+        float dsel = 0.f;                                                 // A[t][t] (v_t . gy_t for GR, GK)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            float a8[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int r = 8 * ks + e;
+                const int sx = 8 * (r / 4) + (r % 4) + dx;                // s - x
+                a8[e] = sx < 0 ? accA[r] : (sx == 0 ? bon : 0.f);
+                if (KIND != SCAN_GV) dsel = sx == 0 ? accA[r] : dsel;
+            }
+            split8(a8, Ah[ks], Al[ks]);
+        }
+        if (KIND != SCAN_GV) {
+            // exactly one lane of each column x holds the diagonal element; both waves computed the same A
+            if (((x >> 2) & 1) == g) L.Diag[x] = dsel;
+        }
+        // ---- MFMA 2: Out[t][o] = sum_s A[t][s] Val[s][o] ----
+        f32x16 accY = {0};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bf16x8 bv = cat8(*reinterpret_cast<const bf16x4*>(&L.VTh[ocol][16 * ks + 4 * g]),
+                                   *reinterpret_cast<const bf16x4*>(&L.VTh[ocol][16 * ks + 8 + 4 * g]));
+            const bf16x8 bvl = cat8(*reinterpret_cast<const bf16x4*>(&L.VTl[ocol][16 * ks + 4 * g]),
+                                    *reinterpret_cast<const bf16x4*>(&L.VTl[ocol][16 * ks + 8 + 4 * g]));
+            accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ah[ks], bv, accY, 0, 0, 0);
+            accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Al[ks], bv, accY, 0, 0, 0);
+            accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ah[ks], bvl, accY, 0, 0, 0);
+            if (LL) accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Al[ks], bvl, accY, 0, 0, 0);
+        }
+        // ---- MFMA 3: Out += Q (rescaled state), the state straight from the accumulators ----
+        const float cr_lane = TT ? (KIND == SCAN_GR ? L.C1[ocol] : L.C3[ocol]) : 0.f;
+#pragma unroll
+        for (int ch2 = 0; ch2 < 2; ++ch2) {
+            const f32x16& S = ch2 == 0 ? S0 : S1;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                float s8[8];
+#pragma unroll
+                for (int e4 = 0; e4 < 2; ++e4) {
+                    f32x4 cr = {cr_lane, cr_lane, cr_lane, cr_lane};
+                    if (!TT) cr = *reinterpret_cast<const f32x4*>(&L.C3[32 * ch2 + 16 * ks + 8 * e4 + 4 * g]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) s8[4 * e4 + e] = S[8 * ks + 4 * e4 + e] * cr[e];
+                }
+                bf16x8 sh, sl;
+                split8(s8, sh, sl);
+                const int c0 = 32 * ch2 + 16 * ks + 4 * g;
+                const bf16x8 ah = cat8(*reinterpret_cast<const bf16x4*>(&L.Qh[x][c0]),
+                                       *reinterpret_cast<const bf16x4*>(&L.Qh[x][c0 + 8]));
+                accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, sh, accY, 0, 0, 0);
+                accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, sl, accY, 0, 0, 0);
+                if (QS) {
+                    const bf16x8 al = cat8(*reinterpret_cast<const bf16x4*>(&L.Ql[x][c0]),
+                                           *reinterpret_cast<const bf16x4*>(&L.Ql[x][c0 + 8]));
+                    accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, sh, accY, 0, 0, 0);
+                    if (LL) accY = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, sl, accY, 0, 0, 0);
+                }
+            }
+        }
+        // ---- MFMA 4: M[c][o] = sum_s Kc[s][c] Val[s][o];  state' = decay * state + scale * M ----
+        const float c2_lane = TT ? L.C2[ocol] : 0.f;
+        const float cu_lane = TT ? (KIND == SCAN_GR ? L.C3[ocol] : L.C1[ocol]) : 0.f;
+#pragma unroll
+        for (int ch2 = 0; ch2 < 2; ++ch2) {
+            f32x16 accM = {0};
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const bf16x8 ah = *reinterpret_cast<const bf16x8*>(&L.KTh[32 * ch2 + x][16 * ks + 8 * g]);
+                const bf16x8 bv = *reinterpret_cast<const bf16x8*>(&L.VTh[ocol][16 * ks + 8 * g]);
+                const bf16x8 bvl = *reinterpret_cast<const bf16x8*>(&L.VTl[ocol][16 * ks + 8 * g]);
+                accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bv, accM, 0, 0, 0);
+                accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bvl, accM, 0, 0, 0);
+                if (KS) {
+                    const bf16x8 al = *reinterpret_cast<const bf16x8*>(&L.KTl[32 * ch2 + x][16 * ks + 8 * g]);
+                    accM = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bv, accM, 0, 0, 0);
+                }
+            }
+            f32x16& S = ch2 == 0 ? S0 : S1;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                f32x4 c2 = {c2_lane, c2_lane, c2_lane, c2_lane}, cu = {cu_lane, cu_lane, cu_lane, cu_lane};
+                if (!TT) {
+                    c2 = *reinterpret_cast<const f32x4*>(&L.C2[32 * ch2 + 8 * r4 + 4 * g]);
+                    cu = *reinterpret_cast<const f32x4*>(&L.C1[32 * ch2 + 8 * r4 + 4 * g]);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + cu[e] * accM[4 * r4 + e];
+            }
+        }
+        // ================================== epilogue ==================================
+        if (KIND == SCAN_GV) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rso, row_off(cc, r, Cs, 4), 0);
+        } else {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");       // Diag: written and read inside a wave
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            float dd[16];                                                         // GK: a - b per row
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const f32x4 dg = *reinterpret_cast<const f32x4*>(&L.Diag[8 * r4 + 4 * g]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * r4 + e;
+                    const int rho = 8 * r4 + 4 * g + e;
+                    const float post = L.Post[rho][ocol];
+                    const float rr = cvt(rraw[r]), kk = cvt(kraw[r]);
+                    const float px = post * accY[r];
+                    if (KIND == SCAN_GR) {
+                        const float gr = fmaf(u_o * kk, dg[e], px);
+                        BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + gr), rso, row_off(cc, r, Cs, 4), 0);
+                        BufRaw<4>::st(__builtin_bit_cast(unsigned, rr * px), rsa, row_off(cc, r, Cs, 4), 0);
+                        gu_acc = fmaf(rr * kk, dg[e], gu_acc);
+                    } else {
+                        const float gk = fmaf(u_o * rr, dg[e], px);
+                        BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + gk), rso, row_off(cc, r, Cs, 4), 0);
+                        dd[r] = __builtin_bit_cast(float, araw[r]) - kk * px;     // rows past T: a = 0, k = 0
+                    }
+                }
+            }
+            if (KIND == SCAN_GK) {
+                // gw_n = ld_n (sum over the tokens scanned before n of (a - b)  -  b_n): a running sum over the
+                // scan rows.  A lane holds rows 8 r4 + 4g + e; its partner (lane ^ 32) the other half of each 8.
+                float bs[4], pbs[4];
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    bs[r4] = (dd[4 * r4] + dd[4 * r4 + 1]) + (dd[4 * r4 + 2] + dd[4 * r4 + 3]);
+                    pbs[r4] = __shfl_xor(bs[r4], 32);
+                }
+                float before = xcarry;
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    float run = before + (g == 1 ? pbs[r4] : 0.f);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = 4 * r4 + e;
+                        const float kk = cvt(kraw[r]);
+                        const float bn = kk * L.Post[8 * r4 + 4 * g + e][ocol] * accY[r];
+                        const float fw = cvtw(wo[r]);
+                        const float ldn = W_IS_EW ? fw : -__expf(fw);
+                        const float gw = ldn * (run - bn);
+                        BufRaw<4>::st(__builtin_bit_cast(unsigned, __builtin_bit_cast(float, pgw[r]) + gw), rsgw,
+                                      row_off(cc, r, Cs, 4), 0);
+                        run += dd[r];
+                    }
+                    before += bs[r4] + pbs[r4];
+                }
+                xcarry = before;
+            }
+        }
+        lds_barrier();                                                   // (3) LDS is rewritten by the next chunk
+    }
+    if (KIND == SCAN_GR && ASC) {
+        gu_acc += __shfl_xor(gu_acc, 32);
+        if (g == 0) gu_part[(size_t)b * C + h * HN + ocol] = gu_acc;
+    }
+    if (threadIdx.x == 0) todo[bh] = 0;
+}
+
+}  // namespace wkv6_detail
+}  // namespace vrwkv
