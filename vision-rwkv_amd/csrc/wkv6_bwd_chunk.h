@@ -46,7 +46,7 @@ struct __attribute__((aligned(16))) ScanLds {
 
 // DIR 0: ascending pass (bonus u, adds to the outputs).  DIR 1: descending pass (writes them).
 template <typename WT, int KIND, int DIR, bool W_IS_EW>
-__global__ __launch_bounds__(128)
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfloat16* __restrict__ k_,
                           const __hip_bfloat16* __restrict__ v_, const WT* __restrict__ w_,
                           const float* __restrict__ u_, const float* __restrict__ gy_,
@@ -68,6 +68,8 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
 
     const int lane = threadIdx.x & 63;
     const int q = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = q;                                    // name used by the timing hook
+    (void)wave;
     const int g = lane >> 5, x = lane & 31;
     const int bh = blockIdx.x;
     const int b = bh / H, h = bh % H;
@@ -122,6 +124,7 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
         int Cs = C;
         asm volatile("" : "+s"(Cs));                       // keep row offsets out of the loop-invariant scalars
         const int cc = chunk_of(ch);
+        WKV6_STAMP(0);
         // =============================== stage E: elementwise =================================
         // wave q prepares pass indices n = 16q .. 16q+15 of the chunk; lane = channel
         RawIO xraw[16], yraw[16];                          // the two bf16 tensors this scan needs here
@@ -148,7 +151,9 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
 #pragma unroll
         for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
         if (q == 0) L.Tot[lane] = p[15];
+        WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
+        WKV6_STAMP(2);
         const float pref = L.Tot[lane];                                  // P_15
         const float off = q == 1 ? pref : 0.f;
         if (q == 1) {
@@ -162,14 +167,15 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
         {
             bf16x8 kth[2], ktl[2], vth[2], vtl[2];
             float pu[16];
+            const int r0 = REV ? 16 * (1 - q) : 16 * q;                   // first scan row of this wave's block
 #pragma unroll
             for (int m = 0; m < 16; ++m) {
                 const int n = 16 * q + m;
-                const int rho = REV ? LC - 1 - n : n;
-                const int e = REV ? 15 - m : m;                           // position inside this wave's 16 rows
+                const int e = REV ? 15 - m : m;                           // position inside this wave's 16 scan rows
+                const int rho = r0 + e;                                   // = n, or 31 - n for a reversed scan
                 const bool ok = token_of_n(cc, n) < T;
                 const float P = p[m] + off;
-                const float f1 = __expf(P - ld[m] - pref);               // exp(Pex - Pref)
+                const float f1 = __expf((m ? p[m - 1] : 0.f) + off - pref);  // exp(Pex - Pref), Pex_m = P_(m-1)
                 const float f2 = __expf(pref - P);                        // exp(Pref - P)
                 const float xa = ok ? cvt(xraw[m]) : 0.f, ya = ok ? cvt(yraw[m]) : 0.f;
                 const float gyv = ok ? __builtin_bit_cast(float, graw[m]) : 0.f;
@@ -191,7 +197,6 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 vth[e >> 3][e & 7] = vh;
                 vtl[e >> 3][e & 7] = (__bf16)(valv - (float)vh);
             }
-            const int r0 = REV ? 16 * (1 - q) : 16 * q;                   // first scan row of this wave's block
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 *reinterpret_cast<bf16x8*>(&L.KTh[lane][r0 + 8 * e]) = kth[e];
@@ -202,11 +207,12 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
             if (KIND == SCAN_GV && ASC) {                                 // bonus_n = sum_j r_n[j] u[j] k_n[j]
                 int idx;
                 const float rs = row_sums16(pu, lane, idx);
-                const int n = 16 * q + idx;
-                L.Bon[lane >> 4][REV ? LC - 1 - n : n] = rs;
+                L.Bon[lane >> 4][r0 + (REV ? 15 - idx : idx)] = rs;
             }
         }
+        WKV6_STAMP(3);
         lds_barrier();                                                   // (2)
+        WKV6_STAMP(4);
         if (sFlag) {                                                      // out of range: left to the sequential kernels
             if (threadIdx.x == 0) todo[bh] = 1;
             return;
@@ -221,15 +227,10 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
         RawW wo[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
+            if (KIND != SCAN_GK) prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
             if (KIND != SCAN_GV) {
                 rraw[r] = BufRaw<2>::ld(rsr, row_off(cc, r, Cs, 2), 0);
                 kraw[r] = BufRaw<2>::ld(rsk, row_off(cc, r, Cs, 2), 0);
-            }
-            if (KIND == SCAN_GK) {
-                araw[r] = BufRaw<4>::ld(rsa, row_off(cc, r, Cs, 4), 0);
-                wo[r] = BufRaw<sizeof(WT)>::ld(rsw, row_off(cc, r, Cs, sizeof(WT)), 0);
-                pgw[r] = ASC ? BufRaw<4>::ld(rsgw, row_off(cc, r, Cs, 4), 0) : 0u;
             }
         }
         // ---- MFMA 1: A^T: acc[s][t] = sum_c Kc[s][c] Q[t][c]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
@@ -312,6 +313,15 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 }
             }
         }
+        if (KIND == SCAN_GK) {                                            // late: these would not fit beside MFMA 1-3
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                araw[r] = BufRaw<4>::ld(rsa, row_off(cc, r, Cs, 4), 0);
+                wo[r] = BufRaw<sizeof(WT)>::ld(rsw, row_off(cc, r, Cs, sizeof(WT)), 0);
+                prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
+                pgw[r] = ASC ? BufRaw<4>::ld(rsgw, row_off(cc, r, Cs, 4), 0) : 0u;
+            }
+        }
         // ---- MFMA 4: M[c][o] = sum_s Kc[s][c] Val[s][o];  state' = decay * state + scale * M ----
         const float c2_lane = TT ? L.C2[ocol] : 0.f;
         const float cu_lane = TT ? (KIND == SCAN_GR ? L.C3[ocol] : L.C1[ocol]) : 0.f;
@@ -342,6 +352,7 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + cu[e] * accM[4 * r4 + e];
             }
         }
+        WKV6_STAMP(5);
         // ================================== epilogue ==================================
         if (KIND == SCAN_GV) {
 #pragma unroll
@@ -403,7 +414,9 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 xcarry = before;
             }
         }
+        WKV6_STAMP(6);
         lds_barrier();                                                   // (3) LDS is rewritten by the next chunk
+        WKV6_STAMP(7);
     }
     if (KIND == SCAN_GR && ASC) {
         gu_acc += __shfl_xor(gu_acc, 32);

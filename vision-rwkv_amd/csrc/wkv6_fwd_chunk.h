@@ -227,7 +227,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             for (int m = 0; m < 16; ++m) {
                 const int n = 16 * q + m;
                 const float P = p[m] + off;
-                const float f1 = __expf(P - ld[m] - pref);               // exp(Pex - Pref)
+                const float f1 = __expf((m ? p[m - 1] : 0.f) + off - pref);  // exp(Pex - Pref), Pex_m = P_(m-1)
                 const float f2 = __expf(pref - P);                        // exp(Pref - P)
                 const float rt = rr[m] * f1, kt = kk[m] * f2;
                 const __bf16 rh = (__bf16)rt, kh = (__bf16)kt;
