@@ -73,7 +73,8 @@ int vrwkv_biwkv_bwd(const float* w, const float* u, const void* k, const void* v
  * w_is_ew = 0: w is the raw decay logit and the kernel uses d = exp(-exp(w)), i.e. it folds in
  *              the `ew = -exp(w)` of WKV_6.forward (vrwkv6.py:48);
  * w_is_ew = 1: w already holds ew = -exp(w_raw), as the reference extension receives it.
- * State and accumulation are fp32.  No limit on T. */
+ * State and accumulation are fp32.  No limit on T (T*C < 2^29).  No workspace is needed: the size
+ * function returns 0 and workspace may be NULL (both kept so that every operator has the same shape). */
 size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H);
 int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, const float* u,
                    float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
