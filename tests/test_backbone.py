@@ -97,3 +97,45 @@ def test_backbone_trains_through_the_hip_operators():
     out.square().mean().backward()
     g = net.layers[0].att.spatial_decay.grad
     assert g is not None and torch.isfinite(g).all() and g.abs().sum().item() > 0
+
+
+def test_multihead_shift_tensor_ops_match_index_loops():
+    """CPU: per-head Q-Shift by folding heads into the batch, against the index-loop oracle (with and without
+    the trailing class token)."""
+    import vision_rwkv_amd as ops
+    from oracle import qshift
+    rng = np.random.default_rng(3)
+    for cls in (False, True):
+        x = rng.standard_normal((2, 4 * 3 + int(cls), 128)).astype(np.float32)
+        got = ops.q_shift_multihead(torch.from_numpy(x), 1, 64, (4, 3), with_cls_token=cls).numpy()
+        assert np.array_equal(got, qshift.q_shift_multihead_loops(x, 1, 64, (4, 3), with_cls_token=cls))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cls", [False, True])
+def test_vrwkv6_backbone_fused_equals_eager_and_trains(cls):
+    import vision_rwkv_amd as ops
+    torch.manual_seed(2)
+    net = ops.VRWKV6(img_size=64, embed_dims=128, num_heads=2, depth=2, post_norm=True, init_values=0.1,
+                     with_cls_token=cls, output_cls_token=cls).cuda()
+    img = torch.randn(2, 3, 96, 64).cuda()
+    net.eval()
+    with torch.no_grad():
+        y_fused = net(img)
+        for m in net.modules():
+            if hasattr(m, "fused_shift"):
+                m.fused_shift = False
+        y_eager = net(img)
+    fm = y_fused[0] if cls else y_fused
+    fe = y_eager[0] if cls else y_eager
+    assert tuple(fm.shape) == (2, 128, 6, 4)
+    assert (fm - fe).abs().max().item() <= 1e-5
+    if cls:
+        assert tuple(y_fused[1].shape) == (2, 128) and (y_fused[1] - y_eager[1]).abs().max().item() <= 1e-5
+    net.train()
+    out = net(img)
+    (out[0] if cls else out).square().mean().backward()
+    for name in ("time_decay", "time_faaaa", "time_maa_w1"):
+        g = getattr(net.layers[0].att, name).grad
+        assert g is not None and torch.isfinite(g).all(), name
+    assert net.layers[0].att.time_faaaa.grad.abs().sum().item() > 0

@@ -7,5 +7,6 @@ from ._lib import VrwkvError, LIB_PATH, build, lib
 from .ops import WKV, RUN_CUDA, bi_wkv_forward, bi_wkv_backward, WKV_6, RUN_CUDA_RWKV6, wkv6_forward, wkv6_backward, HEAD_SIZE, q_shift, q_shift_mix
 
 from .backbone import VRWKV, vrwkv_l
+from .backbone6 import VRWKV6, vrwkv6_b, q_shift_multihead
 
-__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "wkv6_backward", "HEAD_SIZE", "q_shift", "q_shift_mix", "VRWKV", "vrwkv_l", "VrwkvError", "LIB_PATH", "build", "lib"]
+__all__ = ["WKV", "RUN_CUDA", "bi_wkv_forward", "bi_wkv_backward", "WKV_6", "RUN_CUDA_RWKV6", "wkv6_forward", "wkv6_backward", "HEAD_SIZE", "q_shift", "q_shift_mix", "VRWKV", "vrwkv_l", "VRWKV6", "vrwkv6_b", "q_shift_multihead", "VrwkvError", "LIB_PATH", "build", "lib"]
