@@ -8,6 +8,7 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--io fp32|bf16] [--no-cpu-baseline]
 """
 import argparse
+import math
 import json
 import os
 import sys
@@ -138,6 +139,40 @@ def backward_section(torch, ops, steps, warmup):
             "wkv6_bwd_us_per_call": round(us_6, 1), "wkv6_bwd_tokens_per_s": round(B * T / (us_6 * 1e-6), 1)}
 
 
+def sweep_section(torch, ops, steps, warmup):
+    """Dense-prediction caller shapes (adapter backbones run groups of blocks at T = H/16 * W/16 with batch 2):
+    Bi-WKV forward and backward, fp32 I/O, per (T, C)."""
+    dev = torch.device("cuda:0")
+    rows = []
+    for Tn in (1024, 4150, 4200):
+        for Cn in (192, 384, 768, 1024):
+            Bn = 2
+            g = torch.Generator(device="cpu").manual_seed(Tn + Cn)
+            k, v, gy = (torch.randn(Bn, Tn, Cn, generator=g).to(dev) for _ in range(3))
+            c = torch.arange(Cn, dtype=torch.float32)
+            w = ((-5 + 8 * c / (Cn - 1)) / Tn).to(dev)
+            u = ((math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / Tn).to(dev)
+
+            def timed(fn):
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(steps):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) * 1e3 / steps
+
+            us_f = timed(lambda: ops.bi_wkv_forward(w, u, k, v))
+            us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
+            el = Bn * Tn * Cn * 4
+            rows.append({"B": Bn, "T": Tn, "C": Cn, "fwd_us": round(us_f, 1), "fwd_GBps": round(3 * el / us_f / 1e3, 1),
+                         "bwd_us": round(us_b, 1), "bwd_GBps": round(5 * el / us_b / 1e3, 1)})
+    return rows
+
+
 def backbone_section(torch, ops, steps, warmup):
     """VRWKV-L forward (24 blocks, C=1024, 384x384 input -> T=576) at batch 32 in bf16, random weights:
     ms per forward, and the share of it spent in the 24 Bi-WKV calls (timed alone at the same shape)."""
@@ -171,10 +206,23 @@ def backbone_section(torch, ops, steps, warmup):
         v = torch.randn(Bn, Tn, Cn, device=dev, dtype=torch.bfloat16)
         w, u = (att.spatial_decay / Tn).float(), (att.spatial_first / Tn).float()
         ms_wkv = timed(lambda: ops.bi_wkv_forward(w, u, k, v), 24 * steps, 24 * warmup) * 24
+        # VRWKV6-B at its training shape (batch 64, 224x224 -> T=196, C=768, 12 heads, 12 blocks)
+        B6, H6 = 64, 12
+        net6 = ops.vrwkv6_b().to(dev).eval().bfloat16()
+        img6 = torch.randn(B6, 3, 224, 224, device=dev, dtype=torch.bfloat16)
+        ms6 = timed(lambda: net6(img6), steps, warmup)
+        r6, k6, v6 = (torch.randn(B6, 196, 768, device=dev, dtype=torch.bfloat16) for _ in range(3))
+        w6 = torch.randn(B6, 196, 768, device=dev) * 0.5 - 0.5
+        u6 = torch.randn(H6, 64, device=dev) * 0.1
+        ms_wkv6 = timed(lambda: ops.wkv6_forward(B6, 196, 768, H6, r6, k6, v6, w6, u6), 12 * steps, 12 * warmup) * 12
     return {"workload": f"VRWKV-L forward, batch {Bn}, {S}x{S}, T={Tn}, C={Cn}, 24 blocks, bf16, random weights",
             "ms_per_forward": round(ms_fwd, 3), "images_per_s": round(Bn / ms_fwd * 1e3, 1),
             "ms_per_forward_unfused_shift": round(ms_fwd_eager_shift, 3),
-            "biwkv_ms_per_forward": round(ms_wkv, 3), "biwkv_share": round(ms_wkv / ms_fwd, 4)}
+            "biwkv_ms_per_forward": round(ms_wkv, 3), "biwkv_share": round(ms_wkv / ms_fwd, 4),
+            "vrwkv6_b": {"workload": "VRWKV6-B forward, batch 64, 224x224, T=196, C=768, 12 heads, 12 blocks, bf16, "
+                                     "random weights",
+                         "ms_per_forward": round(ms6, 3), "images_per_s": round(B6 / ms6 * 1e3, 1),
+                         "wkv6_ms_per_forward": round(ms_wkv6, 3), "wkv6_share": round(ms_wkv6 / ms6, 4)}}
 
 
 def main():
@@ -187,6 +235,7 @@ def main():
     ap.add_argument("--no-wkv6", action="store_true", help="skip the secondary wkv6 measurement")
     ap.add_argument("--no-backbone", action="store_true", help="skip the VRWKV-L whole-forward measurement")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-kernel measurements")
+    ap.add_argument("--sweep", action="store_true", help="also time Bi-WKV at the dense-prediction shapes (B=2, long T)")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -290,6 +339,8 @@ def main():
         out["wkv6"] = wkv6_section(torch, ops, max(args.steps, 10), max(args.warmup // 5, 3), not args.no_cpu_baseline)
     if not args.no_backward:
         out["backward"] = backward_section(torch, ops, 10, 3)
+    if args.sweep:
+        out["sweep"] = sweep_section(torch, ops, 10, 3)
     if not args.no_backbone:
         out["backbone"] = backbone_section(torch, ops, 5, 3)
     print(json.dumps(out))

@@ -78,7 +78,7 @@ BwdPlan make_bwd_plan(int B, int T, int C) {
     }
     p.planes = (size_t)5 * B * T * C;                        // sequential form: 5 floats per element
     p.agg1 = (size_t)B * p.nSC * 5 * C;
-    p.agg2 = (size_t)B * p.nSC * BWD_SMAX * 9 * C;
+    p.agg2 = (size_t)B * p.nSC * 8 * C;
     p.parts = (size_t)2 * B * p.nSC * C;
     p.total = p.planes + p.agg1 + p.agg2 + p.parts;
     return p;

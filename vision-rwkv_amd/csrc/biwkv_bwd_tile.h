@@ -77,7 +77,7 @@ struct ZScan {
 
 // Auxiliary table of the long-sequence path (floats):
 //   agg1 [B][nSC][5][C]      forward aggregates of a super-chunk at its own scale R: A, B, R, Cg, D
-//   agg2 [B][nSC][8][9][C]   per wave: past-side sums (s0, s1, l0, l1), future-side sums, scale Re
+//   agg2 [B][nSC][8][C]      z-sums of a super-chunk at the common scale 2^-R: past side (s0, s1, l0, l1), future side
 struct BwdGeom {
     int n_ctile, nSC, n_tiles;      // tile id = (b * nSC + sc) * n_ctile + ctile
 };
@@ -118,9 +118,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         if (!bwd_tile_is_fast(om, mu, T)) continue;          // workgroup-uniform: same channels in every wave
         const int cc = cok ? c0 : 0;                         // in-range column for the auxiliary table
         auto a1 = [&](int s, int slot) -> float& { return agg1[(((size_t)b * nSC + s) * 5 + slot) * C + cc]; };
-        auto a2 = [&](int s, int wv, int slot) -> float& {
-            return agg2[((((size_t)b * nSC + s) * BWD_SMAX + wv) * 9 + slot) * C + cc];
-        };
+        auto a2 = [&](int s, int slot) -> float& { return agg2[(((size_t)b * nSC + s) * 8 + slot) * C + cc]; };
 
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes);
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
@@ -172,7 +170,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         s1[wave][4][lane] = Dg;
         lds_barrier();
 
-        float a = 0.f, bb = 0.f, c = 0.f, d = 0.f, Re;
+        float a = 0.f, bb = 0.f, c = 0.f, d = 0.f, Re, Rw_to_R;
         {
             float la[BWD_SMAX], lb[BWD_SMAX], lc[BWD_SMAX], ld[BWD_SMAX], lr[BWD_SMAX];
 #pragma unroll
@@ -238,6 +236,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                     c = fmaf(G, c, ldexpf(lc[s], sh));
                     d = fmaf(G, d, ldexpf(ld[s], sh));
                 }
+            Rw_to_R = r - Rw;
             const float upf = fminf(r - Rw, 100.f);
             const int up = (int)upf;
             a = ldexpf(a, up); bb = ldexpf(bb, up); c = ldexpf(c, up); d = ldexpf(d, up);
@@ -274,12 +273,30 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         for (int j = 0; j < L; ++j) pl.push(gd, Z[j], ZY[j]);
 
         if (MODE == 2) {
-            if (cok) {
-                a2(sc, wave, 0) = pl.s0; a2(sc, wave, 1) = pl.s1; a2(sc, wave, 2) = pl.l0; a2(sc, wave, 3) = pl.l1;
-                a2(sc, wave, 4) = fl.s0; a2(sc, wave, 5) = fl.s1; a2(sc, wave, 6) = fl.l0; a2(sc, wave, 7) = fl.l1;
-                a2(sc, wave, 8) = Re;
+            // fold the waves' z-sums into one entry per super-chunk at the sequence's common scale 2^-R
+            // (z 2^R = gy / (D 2^-R) stays within |gy| 2^+-50 under the plain-sum bound, so this is safe)
+            s2[wave][0][lane] = pl.s0; s2[wave][1][lane] = pl.s1; s2[wave][2][lane] = pl.l0; s2[wave][3][lane] = pl.l1;
+            s2[wave][4][lane] = fl.s0; s2[wave][5][lane] = fl.s1; s2[wave][6][lane] = fl.l0; s2[wave][7][lane] = fl.l1;
+            s2[wave][8][lane] = Re;
+            lds_barrier();
+            if (wave == 0 && cok) {
+                const float Rg = Re + fminf(Rw_to_R, 100.f);                  // = R (Re = R - min(R - Rw, 100))
+                ZScan ps, fs;
+                const float nL = (float)L;
+                for (int sw = 0; sw < S; ++sw) {
+                    const int sh = shift_of(Rg - s2[sw][8][lane]);
+                    ps.hop(G, nL, ldexpf(s2[sw][0][lane], sh), ldexpf(s2[sw][1][lane], sh),
+                           ldexpf(s2[sw][2][lane], sh), ldexpf(s2[sw][3][lane], sh));
+                }
+                for (int sw = S - 1; sw >= 0; --sw) {
+                    const int sh = shift_of(Rg - s2[sw][8][lane]);
+                    fs.hop(G, nL, ldexpf(s2[sw][4][lane], sh), ldexpf(s2[sw][5][lane], sh),
+                           ldexpf(s2[sw][6][lane], sh), ldexpf(s2[sw][7][lane], sh));
+                }
+                a2(sc, 0) = ps.s0; a2(sc, 1) = ps.s1; a2(sc, 2) = ps.l0; a2(sc, 3) = ps.l1;
+                a2(sc, 4) = fs.s0; a2(sc, 5) = fs.s1; a2(sc, 6) = fs.l0; a2(sc, 7) = fs.l1;
             }
-            lds_barrier();                                    // s1 is rewritten by the next tile
+            lds_barrier();                                    // s1, s2 are rewritten by the next tile
             continue;
         }
 
@@ -293,19 +310,13 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         {
             const float nL = (float)L;
             if (MODE == 3) {
-                // every wave of the other super-chunks, nearest last (they all span L token positions)
-                for (int s = 0; s < sc; ++s)
-                    for (int wv = 0; wv < BWD_SMAX; ++wv) {
-                        const int sh = shift_of(Rw - a2(s, wv, 8));
-                        p.hop(G, nL, ldexpf(a2(s, wv, 0), sh), ldexpf(a2(s, wv, 1), sh),
-                              ldexpf(a2(s, wv, 2), sh), ldexpf(a2(s, wv, 3), sh));
-                    }
-                for (int s = nSC - 1; s > sc; --s)
-                    for (int wv = BWD_SMAX - 1; wv >= 0; --wv) {
-                        const int sh = shift_of(Rw - a2(s, wv, 8));
-                        f.hop(G, nL, ldexpf(a2(s, wv, 4), sh), ldexpf(a2(s, wv, 5), sh),
-                              ldexpf(a2(s, wv, 6), sh), ldexpf(a2(s, wv, 7), sh));
-                    }
+                // the other super-chunks (their sums are at the common scale 2^-R), nearest last; then to my scale
+                const float GS = fast_exp2(-om * (float)(S * L)), nSL = (float)(S * L);
+                for (int s = 0; s < sc; ++s) p.hop(GS, nSL, a2(s, 0), a2(s, 1), a2(s, 2), a2(s, 3));
+                for (int s = nSC - 1; s > sc; --s) f.hop(GS, nSL, a2(s, 4), a2(s, 5), a2(s, 6), a2(s, 7));
+                const int sh = shift_of(-Rw_to_R);                        // 2^(Rw - R) <= 1
+                p.s0 = ldexpf(p.s0, sh); p.s1 = ldexpf(p.s1, sh); p.l0 = ldexpf(p.l0, sh); p.l1 = ldexpf(p.l1, sh);
+                f.s0 = ldexpf(f.s0, sh); f.s1 = ldexpf(f.s1, sh); f.l0 = ldexpf(f.l0, sh); f.l1 = ldexpf(f.l1, sh);
             }
 #pragma unroll
             for (int s = 0; s < BWD_SMAX; ++s)
