@@ -101,7 +101,10 @@ struct TileGeom {
 
 // MODE 0: whole sequence in one workgroup.  MODE 1: aggregate-only pass of the long-
 // sequence path (writes the workspace).  MODE 2: emit pass of the long-sequence path.
-template <typename IO, int VEC, int L, int MODE>
+// STAGED (fp32 I/O, C % 4 == 0, 16-byte aligned k, v): a tile's k, v rows are fetched as 16-byte pieces straight
+// into LDS (buffer_load ... lds, no registers, 1 KB contiguous per wave instruction instead of 256 B) while the
+// previous tile is computed, and each wave then reads its own rows back lane-per-channel.
+template <typename IO, int VEC, int L, int MODE, bool STAGED = false>
 struct BiwkvTile {
     static constexpr int SMAX = smax_for(L, VEC);
     static constexpr int CH = WAVE * VEC;
@@ -118,6 +121,7 @@ struct BiwkvTile {
     TileGeom g;
     int lane, wave, S;
     AggPtr s_agg0, s_agg1;      // two LDS exchange buffers, alternated tile by tile
+    float* s_stage;             // STAGED: this wave's [2][L][64] floats of LDS (k rows, then v rows)
 
     struct Where {
         int b, sc, ctile, c0, tw;
@@ -170,6 +174,25 @@ struct BiwkvTile {
         }
     }
 
+    // STAGED: this wave's L rows of k and v of `tile`, 4 rows per instruction (lane = row l/16, channels 4(l%16)..+3),
+    // land in s_stage as [row][64 channels]; rows past T and channels past C are dropped by the range check.
+    __device__ __forceinline__ void issue_stage(int tile, WU& wu) const {
+        issue_wu(tile, wu);
+        const Where q = locate(tile);
+        const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + q.slab, bytes);
+        const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + q.slab, bytes);
+        const int cq = q.ctile * WAVE + (lane & 15) * 4;
+#pragma unroll
+        for (int i = 0; i < L / 4; ++i) {
+            const int row = q.tw + 4 * i + (lane >> 4);
+            const unsigned vo = (row < T && cq < C) ? (unsigned)(((size_t)row * C + cq) * sizeof(float)) : OOB_OFFSET;
+            typedef __attribute__((address_space(3))) void* lds_ptr;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)(s_stage + i * 256), 16, vo, 0, 0, CPOL_NT);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(s_stage + L * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
+        }
+    }
+
     // Computes one tile from the packed registers K, V; in the middle (once K, V have been
     // consumed) issues the loads of `next` into Kn, Vn when next < n_tiles.
     // True when any channel of the tile is outside the plain-sum regime (wave-uniform, and the
@@ -205,7 +228,14 @@ struct BiwkvTile {
 
         float om[VEC], mu[VEC];
         if (tile_is_robust(wu, om, mu)) {
-            if (next < g.n_tiles) issue_loads(next, Kn, Vn, wun);
+            if (next < g.n_tiles) {
+                if (STAGED) {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the skipped tile's rows must have landed
+                    issue_stage(next, wun);
+                } else {
+                    issue_loads(next, Kn, Vn, wun);
+                }
+            }
             return;
         }
 
@@ -218,7 +248,7 @@ struct BiwkvTile {
         // The next tile is fetched a token at a time behind the arithmetic (k during the
         // aggregate pass, v during the ascending sweep): few vector-memory instructions are
         // outstanding per CU at any moment, so issuing them never stalls the wave for long.
-        const bool have_next = next < g.n_tiles;
+        const bool have_next = next < g.n_tiles && !STAGED;          // register prefetch of the next tile
         const Where qn = locate(have_next ? next : tile);
         const __amdgpu_buffer_rsrc_t rkn = make_rsrc(k_ + qn.slab, (unsigned)((size_t)T * C * sizeof(IO)));
         const __amdgpu_buffer_rsrc_t rvn = make_rsrc(v_ + qn.slab, (unsigned)((size_t)T * C * sizeof(IO)));
@@ -226,13 +256,28 @@ struct BiwkvTile {
 
         // unpack; tokens past T read as zero from the buffer and get k = -inf here
         float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
+        if (STAGED) {
+            // this tile's rows have landed (loads and the previous tile's stores share one counter and may
+            // retire in either order, so the wait is for all of them)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int j = 0; j < L; ++j) {
-            unpack<IO, VEC>(K[j], X0[j]);
-            unpack<IO, VEC>(V[j], X1[j]);
-            const bool tok = q.tw + j < T;               // wave-uniform
+            for (int j = 0; j < L; ++j) {
+                const bool tok = q.tw + j < T;
+                const float kk = s_stage[j * WAVE + lane], vv = s_stage[(L + j) * WAVE + lane];
+                X0[j][0] = tok ? kk : NEG_INF;
+                X1[j][0] = tok ? vv : 0.f;               // rows past T were not written: LDS holds stale bits
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
+            if (next < g.n_tiles) issue_stage(next, wun);
+        } else {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) X0[j][e] = tok ? X0[j][e] : NEG_INF;
+            for (int j = 0; j < L; ++j) {
+                unpack<IO, VEC>(K[j], X0[j]);
+                unpack<IO, VEC>(V[j], X1[j]);
+                const bool tok = q.tw + j < T;               // wave-uniform
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) X0[j][e] = tok ? X0[j][e] : NEG_INF;
+            }
         }
 
         // ================================== fast path ==================================
@@ -287,7 +332,12 @@ struct BiwkvTile {
             s_agg[wave][3][li + e] = Cg[e];
             s_agg[wave][4][li + e] = D[e];
         }
-        lds_barrier();
+        if (STAGED) {
+            // LDS-only barrier by hand: the fence form would also wait for the next tile's staging loads
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else {
+            lds_barrier();
+        }
 
         float G[VEC];                                     // decay over one wave's chunk
 #pragma unroll
@@ -553,14 +603,15 @@ struct BiwkvTile {
 };
 
 
-template <typename IO, int VEC, int L, int MODE>
+template <typename IO, int VEC, int L, int MODE, bool STAGED = false>
 __global__ __launch_bounds__(smax_for(L, VEC) * WAVE)
 void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
                       const IO* __restrict__ k_, const IO* __restrict__ v_, IO* __restrict__ y_,
                       float* __restrict__ ws, int T, int C, TileGeom g)
 {
-    using Tile = BiwkvTile<IO, VEC, L, MODE>;
+    using Tile = BiwkvTile<IO, VEC, L, MODE, STAGED>;
     __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
+    __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? Tile::SMAX : 1][2][STAGED ? L : 1][WAVE];
 
     Tile t;
     t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
@@ -570,12 +621,13 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     t.S = blockDim.x >> 6;
     t.s_agg0 = s_agg[0];
     t.s_agg1 = s_agg[1];
+    t.s_stage = &s_stage[STAGED ? t.wave : 0][0][0][0];
 
     typename Tile::P K0[L], V0[L], K1[L], V1[L];
     typename Tile::WU wu0, wu1;
     int tile = blockIdx.x;
     if (tile >= g.n_tiles) return;
-    t.issue_loads(tile, K0, V0, wu0);
+    if (STAGED) t.issue_stage(tile, wu0); else t.issue_loads(tile, K0, V0, wu0);
     for (;;) {
         int next = tile + gridDim.x;
         t.run(tile, next, 0, K0, V0, wu0, K1, V1, wu1);
@@ -666,6 +718,14 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
     const IO* vv = static_cast<const IO*>(v);
     IO* yy = static_cast<IO*>(y);
     if (!p.multi()) {
+        if constexpr (sizeof(IO) == 4 && VEC == 1 && L % 4 == 0) {
+            // rows staged through LDS in 16-byte pieces when the layout allows it
+            const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
+            if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
+                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+                return check_launch("biwkv_fwd");
+            }
+        }
         hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
     } else {
         hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
