@@ -96,6 +96,15 @@ void launch_tiled(const BwdPlan& p, const float* w, const float* u, const IO* k,
     if (grid > geo.n_tiles) grid = geo.n_tiles;
     const dim3 g(grid), blk(p.S * WAVE);
     if (p.nSC == 1) {
+        if constexpr (sizeof(IO) == 4 && L % 4 == 0) {
+            const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
+            const char* ns = getenv("VRWKV_BIWKV_NO_STAGE");
+            if (aligned && !(ns && atoi(ns))) {
+                hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 0, true>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
+                                   gw_part, gu_part, B, T, C, geo);
+                return;
+            }
+        }
         hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 0>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
                            gw_part, gu_part, B, T, C, geo);
     } else if constexpr (L == 28) {

@@ -82,7 +82,9 @@ struct BwdGeom {
     int n_ctile, nSC, n_tiles;      // tile id = (b * nSC + sc) * n_ctile + ctile
 };
 
-template <typename IO, int L, int MODE>
+// STAGED (MODE 0, fp32 I/O, C % 4 == 0, 16-byte aligned k, v): the next tile's k, v rows are fetched straight into
+// LDS in 16-byte pieces (buffer_load ... lds) while this tile is computed; gy stays a register load.
+template <typename IO, int L, int MODE, bool STAGED = false>
 __global__ __launch_bounds__(BWD_SMAX * WAVE)
 void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
                            const IO* __restrict__ k_, const IO* __restrict__ v_, const IO* __restrict__ gy_,
@@ -95,6 +97,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
     __shared__ float s1[BWD_SMAX][5][WAVE];
     __shared__ float s2[BWD_SMAX][9][WAVE];
     __shared__ float s3[BWD_SMAX][2][WAVE];
+    __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? BWD_SMAX : 1][2][STAGED ? L : 1][WAVE];
 
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -104,6 +107,32 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
     const unsigned row = (unsigned)(C * sizeof(IO));
     const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
     auto shift_of = [](float d) -> int { return (int)fminf(fmaxf(d, -300.f), 300.f); };
+
+    // workgroup barrier that orders LDS traffic only; the staged variant must not use the fence form, which
+    // would also wait for the next tile's staging loads
+    auto wg_barrier = [&]() {
+        if (STAGED) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else lds_barrier();
+    };
+    float* const stage = &s_stage[STAGED ? wave : 0][0][0][0];
+    auto issue_stage = [&](int tile) {                       // this wave's L rows of k and v, 4 rows per instruction
+        const int ctile = tile % n_ctile;
+        const int sc = (tile / n_ctile) % nSC, b = tile / n_ctile / nSC;
+        const int tw = (sc * S + wave) * L;
+        const size_t slab = (size_t)b * T * C;
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes);
+        const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
+        const int cq = ctile * WAVE + (lane & 15) * 4;
+#pragma unroll
+        for (int i = 0; i < L / 4; ++i) {
+            const int rowt = tw + 4 * i + (lane >> 4);
+            const unsigned vo = (rowt < T && cq < C) ? (unsigned)(((size_t)rowt * C + cq) * 4) : OOB_OFFSET;
+            typedef __attribute__((address_space(3))) void* lds_ptr;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)(stage + i * 256), 16, vo, 0, 0, CPOL_NT);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(stage + L * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
+        }
+    };
+    if (STAGED && (int)blockIdx.x < n_tiles) issue_stage(blockIdx.x);
 
     for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int ctile = tile % n_ctile;
@@ -115,7 +144,14 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         const size_t slab = (size_t)b * T * C;
         const float om = (cok ? w_[c0] : 0.f) * LOG2E;
         const float mu = (cok ? u_[c0] : 0.f) * LOG2E;
-        if (!bwd_tile_is_fast(om, mu, T)) continue;          // workgroup-uniform: same channels in every wave
+        const int next_tile = tile + gridDim.x;
+        if (!bwd_tile_is_fast(om, mu, T)) {                   // workgroup-uniform: same channels in every wave
+            if (STAGED && next_tile < n_tiles) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // the skipped tile's rows must have landed
+                issue_stage(next_tile);
+            }
+            continue;
+        }
         const int cc = cok ? c0 : 0;                         // in-range column for the auxiliary table
         auto a1 = [&](int s, int slot) -> float& { return agg1[(((size_t)b * nSC + s) * 5 + slot) * C + cc]; };
         auto a2 = [&](int s, int slot) -> float& { return agg2[(((size_t)b * nSC + s) * 8 + slot) * C + cc]; };
@@ -124,16 +160,29 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
         const __amdgpu_buffer_rsrc_t rg = make_rsrc(gy_ + slab, bytes);
         Raw Kr[L], Vr[L], Gr[L];
+        float Ks[L], Vs[L];
+        if (STAGED) {
+            // this tile's rows have landed (loads and the previous tile's stores share one counter)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int j = 0; j < L; ++j) {
-            const unsigned vo = voff0 + (unsigned)j * row;
-            Kr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rk, vo, 0);
-            Vr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rv, vo, 0);
-        }
-        if (MODE != 1) {
-#pragma unroll
-            for (int j = 0; j < L; ++j)
+            for (int j = 0; j < L; ++j)                      // gy first: it must not queue behind the next tile's rows
                 Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
+#pragma unroll
+            for (int j = 0; j < L; ++j) { Ks[j] = stage[j * WAVE + lane]; Vs[j] = stage[(L + j) * WAVE + lane]; }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
+            if (next_tile < n_tiles) issue_stage(next_tile);
+        } else {
+#pragma unroll
+            for (int j = 0; j < L; ++j) {
+                const unsigned vo = voff0 + (unsigned)j * row;
+                Kr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rk, vo, 0);
+                Vr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rv, vo, 0);
+            }
+            if (MODE != 1) {
+#pragma unroll
+                for (int j = 0; j < L; ++j)
+                    Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
+            }
         }
 
         const float gd = fast_exp2(-om), cu = fast_exp2(mu);
@@ -144,9 +193,9 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         float m = NEG_INF;
 #pragma unroll
         for (int j = 0; j < L; ++j) {
-            const float kk = unpack1<IO>(Kr[j]);
+            const float kk = STAGED ? Ks[j] : unpack1<IO>(Kr[j]);
             E[j] = (tw + j < T) ? kk : NEG_INF;               // tokens past T: k = -inf
-            V[j] = unpack1<IO>(Vr[j]);
+            V[j] = STAGED ? ((tw + j < T) ? Vs[j] : 0.f) : unpack1<IO>(Vr[j]);   // staged rows past T are stale LDS
             m = fmaxf(m, E[j]);
         }
         const bool any = m > NEG_INF;
@@ -168,7 +217,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         s1[wave][2][lane] = any ? Rw : NEG_BIG;
         s1[wave][3][lane] = Cg;
         s1[wave][4][lane] = Dg;
-        lds_barrier();
+        wg_barrier();
 
         float a = 0.f, bb = 0.f, c = 0.f, d = 0.f, Re, Rw_to_R;
         {
@@ -206,7 +255,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                 if (wave == 0 && cok) {
                     a1(sc, 0) = a; a1(sc, 1) = bb; a1(sc, 2) = r; a1(sc, 3) = c; a1(sc, 4) = d;
                 }
-                lds_barrier();                                // s1 is rewritten by the next tile
+                wg_barrier();                                // s1 is rewritten by the next tile
                 continue;
             }
             if (MODE >= 2) {
@@ -278,7 +327,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             s2[wave][0][lane] = pl.s0; s2[wave][1][lane] = pl.s1; s2[wave][2][lane] = pl.l0; s2[wave][3][lane] = pl.l1;
             s2[wave][4][lane] = fl.s0; s2[wave][5][lane] = fl.s1; s2[wave][6][lane] = fl.l0; s2[wave][7][lane] = fl.l1;
             s2[wave][8][lane] = Re;
-            lds_barrier();
+            wg_barrier();
             if (wave == 0 && cok) {
                 const float Rg = Re + fminf(Rw_to_R, 100.f);                  // = R (Re = R - min(R - Rw, 100))
                 ZScan ps, fs;
@@ -296,7 +345,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                 a2(sc, 0) = ps.s0; a2(sc, 1) = ps.s1; a2(sc, 2) = ps.l0; a2(sc, 3) = ps.l1;
                 a2(sc, 4) = fs.s0; a2(sc, 5) = fs.s1; a2(sc, 6) = fs.l0; a2(sc, 7) = fs.l1;
             }
-            lds_barrier();                                    // s1, s2 are rewritten by the next tile
+            wg_barrier();                                    // s1, s2 are rewritten by the next tile
             continue;
         }
 
@@ -304,7 +353,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         s2[wave][0][lane] = pl.s0; s2[wave][1][lane] = pl.s1; s2[wave][2][lane] = pl.l0; s2[wave][3][lane] = pl.l1;
         s2[wave][4][lane] = fl.s0; s2[wave][5][lane] = fl.s1; s2[wave][6][lane] = fl.l0; s2[wave][7][lane] = fl.l1;
         s2[wave][8][lane] = Re;
-        lds_barrier();
+        wg_barrier();
 
         ZScan p, f;
         {
@@ -357,7 +406,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         // partial sums of gw, gu per (b, super-chunk, c): over this wave's tokens, then over the waves
         s3[wave][0][lane] = gw_acc;
         s3[wave][1][lane] = gu_acc;
-        lds_barrier();
+        wg_barrier();
         if (wave == 0 && cok) {
             float sw = 0.f, su = 0.f;
             for (int s = 0; s < S; ++s) { sw += s3[s][0][lane]; su += s3[s][1][lane]; }
