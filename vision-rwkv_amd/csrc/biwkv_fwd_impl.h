@@ -717,15 +717,20 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
     IO* yy = static_cast<IO*>(y);
-    if (!p.multi()) {
-        if constexpr (sizeof(IO) == 4 && VEC == 1 && L % 4 == 0) {
-            // rows staged through LDS in 16-byte pieces when the layout allows it
-            const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
-            if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
+    // fp32 rows are staged through LDS in 16-byte pieces when the layout allows it
+    if constexpr (sizeof(IO) == 4 && VEC == 1 && L % 4 == 0) {
+        const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
+        if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
+            if (!p.multi()) {
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
-                return check_launch("biwkv_fwd");
+            } else {
+                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
             }
+            return check_launch("biwkv_fwd");
         }
+    }
+    if (!p.multi()) {
         hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
     } else {
         hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
