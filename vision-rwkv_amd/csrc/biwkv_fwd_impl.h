@@ -101,7 +101,7 @@ struct TileGeom {
 
 // MODE 0: whole sequence in one workgroup.  MODE 1: aggregate-only pass of the long-
 // sequence path (writes the workspace).  MODE 2: emit pass of the long-sequence path.
-// STAGED (fp32 I/O, C % 4 == 0, 16-byte aligned k, v): a tile's k, v rows are fetched as 16-byte pieces straight
+// STAGED (C a multiple of the 4 or 8 elements in 16 bytes, 16-byte aligned k, v, y): a tile's k, v rows are fetched as 16-byte pieces straight
 // into LDS (buffer_load ... lds, no registers, 1 KB contiguous per wave instruction instead of 256 B) while the
 // previous tile is computed, and each wave then reads its own rows back lane-per-channel.
 template <typename IO, int VEC, int L, int MODE, bool STAGED = false>
@@ -110,6 +110,11 @@ struct BiwkvTile {
     static constexpr int CH = WAVE * VEC;
     using P = Packed<IO, VEC>;
     typedef float (*AggPtr)[NSLOT][CH];
+    // staging geometry: a lane moves 16 bytes = EPL elements; LPR lanes cover a 64-channel row; an instruction RPI rows
+    static constexpr int EPL = 16 / (int)sizeof(IO), LPR = WAVE / EPL, RPI = WAVE / LPR;
+    static constexpr int NI = (L + RPI - 1) / RPI, LR = NI * RPI;         // instructions and LDS rows per tensor
+    static constexpr bool OUT_STAGED = STAGED && sizeof(IO) == 2;         // 16-bit y goes out in 16-byte pieces as well
+    static constexpr int STAGE_ELEMS = (2 + (OUT_STAGED ? 1 : 0)) * LR * WAVE;   // per wave: k rows, v rows, (y rows)
 
     const float* __restrict__ w_;
     const float* __restrict__ u_;
@@ -121,7 +126,7 @@ struct BiwkvTile {
     TileGeom g;
     int lane, wave, S;
     AggPtr s_agg0, s_agg1;      // two LDS exchange buffers, alternated tile by tile
-    float* s_stage;             // STAGED: this wave's [2][L][64] floats of LDS (k rows, then v rows)
+    IO* s_stage;                // STAGED: this wave's LDS rows [LR][64] of k, then v (then y for 16-bit I/O)
 
     struct Where {
         int b, sc, ctile, c0, tw;
@@ -174,7 +179,7 @@ struct BiwkvTile {
         }
     }
 
-    // STAGED: this wave's L rows of k and v of `tile`, 4 rows per instruction (lane = row l/16, channels 4(l%16)..+3),
+    // STAGED: this wave's L rows of k and v of `tile`, RPI rows per instruction (lane = row l/LPR, EPL channels),
     // land in s_stage as [row][64 channels]; rows past T and channels past C are dropped by the range check.
     __device__ __forceinline__ void issue_stage(int tile, WU& wu) const {
         issue_wu(tile, wu);
@@ -182,14 +187,15 @@ struct BiwkvTile {
         const unsigned bytes = (unsigned)((size_t)T * C * sizeof(IO));
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + q.slab, bytes);
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + q.slab, bytes);
-        const int cq = q.ctile * WAVE + (lane & 15) * 4;
+        const int cq = q.ctile * WAVE + (lane % LPR) * EPL;
 #pragma unroll
-        for (int i = 0; i < L / 4; ++i) {
-            const int row = q.tw + 4 * i + (lane >> 4);
-            const unsigned vo = (row < T && cq < C) ? (unsigned)(((size_t)row * C + cq) * sizeof(float)) : OOB_OFFSET;
+        for (int i = 0; i < NI; ++i) {
+            const int rl = RPI * i + lane / LPR;                          // row inside this wave's chunk
+            const int row = q.tw + rl;
+            const unsigned vo = (rl < L && row < T && cq < C) ? (unsigned)(((size_t)row * C + cq) * sizeof(IO)) : OOB_OFFSET;
             typedef __attribute__((address_space(3))) void* lds_ptr;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)(s_stage + i * 256), 16, vo, 0, 0, CPOL_NT);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(s_stage + L * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)(s_stage + i * RPI * WAVE), 16, vo, 0, 0, CPOL_NT);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(s_stage + (LR + i * RPI) * WAVE), 16, vo, 0, 0, CPOL_NT);
         }
     }
 
@@ -263,7 +269,7 @@ struct BiwkvTile {
 #pragma unroll
             for (int j = 0; j < L; ++j) {
                 const bool tok = q.tw + j < T;
-                const float kk = s_stage[j * WAVE + lane], vv = s_stage[(L + j) * WAVE + lane];
+                const float kk = to_f32(s_stage[j * WAVE + lane]), vv = to_f32(s_stage[(LR + j) * WAVE + lane]);
                 X0[j][0] = tok ? kk : NEG_INF;
                 X1[j][0] = tok ? vv : 0.f;               // rows past T were not written: LDS holds stale bits
             }
@@ -463,7 +469,22 @@ struct BiwkvTile {
                 c[e] = fmaf(gd[e], c[e], X1[j][e]);
                 d[e] = fmaf(gd[e], d[e], X0[j][e]);
             }
-            buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
+            if (OUT_STAGED) s_stage[(2 * LR + j) * WAVE + lane] = from_f32<IO>(out[0]);
+            else buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
+        }
+        if (OUT_STAGED) {
+            // y rows of this wave, written lane-per-channel above, leave as 16-byte pieces (RPI rows per store)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            const int cq = q.ctile * WAVE + (lane % LPR) * EPL;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int rl = RPI * i + lane / LPR;
+                const int rowt = q.tw + rl;
+                const unsigned vo = (rl < L && rowt < T && cq < C) ? (unsigned)(((size_t)rowt * C + cq) * sizeof(IO)) : OOB_OFFSET;
+                const BufRaw<16>::type val = *reinterpret_cast<const BufRaw<16>::type*>(s_stage + (2 * LR + rl) * WAVE + (lane % LPR) * EPL);
+                BufRaw<16>::template st<CPOL_NT>(val, ry, vo, 0);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // the y rows are read before the next tile rewrites them
         }
     }
 
@@ -611,7 +632,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
 {
     using Tile = BiwkvTile<IO, VEC, L, MODE, STAGED>;
     __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
-    __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? Tile::SMAX : 1][2][STAGED ? L : 1][WAVE];
+    __shared__ __attribute__((aligned(16))) IO s_stage[STAGED ? Tile::SMAX : 1][STAGED ? Tile::STAGE_ELEMS : 1];
 
     Tile t;
     t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
@@ -621,7 +642,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     t.S = blockDim.x >> 6;
     t.s_agg0 = s_agg[0];
     t.s_agg1 = s_agg[1];
-    t.s_stage = &s_stage[STAGED ? t.wave : 0][0][0][0];
+    t.s_stage = &s_stage[STAGED ? t.wave : 0][0];
 
     typename Tile::P K0[L], V0[L], K1[L], V1[L];
     typename Tile::WU wu0, wu1;
@@ -718,8 +739,8 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
     const IO* vv = static_cast<const IO*>(v);
     IO* yy = static_cast<IO*>(y);
     // fp32 rows are staged through LDS in 16-byte pieces when the layout allows it
-    if constexpr (sizeof(IO) == 4 && VEC == 1 && L % 4 == 0) {
-        const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
+    if constexpr (VEC == 1) {
+        const bool aligned = C % (16 / (int)sizeof(IO)) == 0 && (((uintptr_t)k | (uintptr_t)v | (uintptr_t)y) & 15) == 0;
         if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
             if (!p.multi()) {
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
