@@ -20,7 +20,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes per launch of the fp32 kernel at this shape: rocprofv3 FETCH_SIZE + WRITE_SIZE of this
 # command with --calibrate-copy, each scaled by what it reads for that plain copy of known size.
-MEASURED_TRAFFIC_FP32 = 115_931_000
+MEASURED_TRAFFIC_FP32 = 115_874_000
 LAYERS = 12
 B, T, C = 64, 196, 768
 
