@@ -114,6 +114,21 @@ def test_ragged_shapes(ops, B, T, C):
         assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= TOL_16
 
 
+def test_very_long_sequence_many_super_chunks(ops):
+    """T = 9100 is 41 super-chunks: more than the carry step's on-chip table holds, so it walks the workspace
+    directly; a second channel tile has parameters outside the plain-sum regime (its entries must stay untouched)."""
+    from oracle import clib
+    B, T, C = 1, 9100, 128
+    rng = np.random.default_rng(91)
+    k = rng.standard_normal((B, T, C), dtype=np.float32)
+    v = rng.standard_normal((B, T, C), dtype=np.float32)
+    w = rng.uniform(-5, 3, C).astype(np.float32) / T
+    u = rng.uniform(-1, 1, C).astype(np.float32)
+    w[70] = 3.0
+    y, _, _ = run(ops, w, u, k, v)
+    assert rel_err(y, clib.biwkv_fwd(w, u, k, v)) <= TOL_F32
+
+
 @pytest.mark.parametrize("T", [40, 196, 700])
 def test_robust_path_extreme_parameters(ops, T):
     """|w| and |u| far outside the plain-sum regime, mixed with benign channels."""

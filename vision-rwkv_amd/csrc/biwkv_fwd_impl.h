@@ -260,6 +260,58 @@ struct BiwkvTile {
         const __amdgpu_buffer_rsrc_t rvn = make_rsrc(v_ + qn.slab, (unsigned)((size_t)T * C * sizeof(IO)));
         if (have_next) issue_wu(next, wun);
 
+        auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
+        // MODE 2: what the other super-chunks contribute -- (A, B) of the earlier ones decayed to this super-chunk's first
+        // token, (C, D) of the later ones decayed to its last -- depends on the workspace alone and is folded here, before
+        // the tile's rows are touched.  Entries are fetched eight at a time (one memory round trip per batch instead of
+        // one per super-chunk); each direction keeps its sum at the running maximum of the scales met so far (all scales
+        // are integers, so re-scaling is an exact ldexp), and the two meet the tile's own scale after the exchange.
+        float ra[VEC], rc[VEC], ca[VEC], cb[VEC], cc[VEC], cd[VEC];
+        if (MODE == 2) {
+            constexpr int NB = 8;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float r1 = NEG_BIG, r2 = NEG_BIG, aa = 0.f, ab = 0.f, ac = 0.f, ad = 0.f;
+                if (q.cok) {
+                    const float GS = fast_exp2(-om[e] * (float)(S * L));
+                    for (int s0 = 0; s0 < q.sc; s0 += NB) {
+                        float tr[NB], t0[NB], t1[NB];
+#pragma unroll
+                        for (int i = 0; i < NB; ++i) {
+                            const int se = s0 + i < q.sc ? s0 + i : q.sc - 1;          // wave-uniform
+                            tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 0, e); t1[i] = ws_at(se, 1, e);
+                        }
+#pragma unroll
+                        for (int i = 0; i < NB; ++i)
+                            if (s0 + i < q.sc) {
+                                const float m = fmaxf(r1, tr[i]);
+                                const int so = shift_of(r1, m), sn = shift_of(tr[i], m);
+                                aa = fmaf(GS, ldexpf(aa, so), ldexpf(t0[i], sn));
+                                ab = fmaf(GS, ldexpf(ab, so), ldexpf(t1[i], sn));
+                                r1 = m;
+                            }
+                    }
+                    for (int s0 = nSC - 1; s0 > q.sc; s0 -= NB) {
+                        float tr[NB], t0[NB], t1[NB];
+#pragma unroll
+                        for (int i = 0; i < NB; ++i) {
+                            const int se = s0 - i > q.sc ? s0 - i : q.sc + 1;
+                            tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 3, e); t1[i] = ws_at(se, 4, e);
+                        }
+#pragma unroll
+                        for (int i = 0; i < NB; ++i)
+                            if (s0 - i > q.sc) {
+                                const float m = fmaxf(r2, tr[i]);
+                                const int so = shift_of(r2, m), sn = shift_of(tr[i], m);
+                                ac = fmaf(GS, ldexpf(ac, so), ldexpf(t0[i], sn));
+                                ad = fmaf(GS, ldexpf(ad, so), ldexpf(t1[i], sn));
+                                r2 = m;
+                            }
+                    }
+                }
+                ra[e] = r1; rc[e] = r2; ca[e] = aa; cb[e] = ab; cc[e] = ac; cd[e] = ad;
+            }
+        }
         // unpack; tokens past T read as zero from the buffer and get k = -inf here
         float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
         if (STAGED) {
@@ -348,8 +400,6 @@ struct BiwkvTile {
         float G[VEC];                                     // decay over one wave's chunk
 #pragma unroll
         for (int e = 0; e < VEC; ++e) G[e] = fast_exp2(-om[e] * (float)L);
-        auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
-
         float a[VEC], bb[VEC], c[VEC], d[VEC], R[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -367,10 +417,7 @@ struct BiwkvTile {
             float r = NEG_BIG;
 #pragma unroll
             for (int s = 0; s < SMAX; ++s) r = fmaxf(r, lr[s]);
-            if (MODE == 2) {
-                r = NEG_BIG;
-                if (q.cok) for (int s = 0; s < nSC; ++s) r = fmaxf(r, ws_at(s, 2, e));
-            }
+            if (MODE == 2) r = fmaxf(r, fmaxf(ra[e], rc[e]));
             r = (r > NEG_BIG) ? r : 0.f;
             R[e] = r;
             float aa = 0.f, ab = 0.f, ac = 0.f, ad = 0.f;
@@ -391,18 +438,9 @@ struct BiwkvTile {
                         ad = fmaf(G[e], ad, ldexpf(ld[s], sh));
                     }
             } else {
-                if (MODE == 2 && q.cok) {
-                    const float GS = fast_exp2(-om[e] * (float)(S * L));
-                    for (int s = 0; s < q.sc; ++s) {
-                        const int sh = shift_of(ws_at(s, 2, e), r);
-                        aa = fmaf(GS, aa, ldexpf(ws_at(s, 0, e), sh));
-                        ab = fmaf(GS, ab, ldexpf(ws_at(s, 1, e), sh));
-                    }
-                    for (int s = nSC - 1; s > q.sc; --s) {
-                        const int sh = shift_of(ws_at(s, 2, e), r);
-                        ac = fmaf(GS, ac, ldexpf(ws_at(s, 3, e), sh));
-                        ad = fmaf(GS, ad, ldexpf(ws_at(s, 4, e), sh));
-                    }
+                if (MODE == 2) {
+                    const int s1 = shift_of(ra[e], r), s2 = shift_of(rc[e], r);
+                    aa = ldexpf(ca[e], s1); ab = ldexpf(cb[e], s1); ac = ldexpf(cc[e], s2); ad = ldexpf(cd[e], s2);
                 }
 #pragma unroll
                 for (int s = 0; s < SMAX; ++s)
