@@ -97,6 +97,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
     __shared__ float s1[BWD_SMAX][5][WAVE];
     __shared__ float s2[BWD_SMAX][9][WAVE];
     __shared__ float s3[BWD_SMAX][2][WAVE];
+    __shared__ float s_in[MODE >= 2 ? BWD_SMAX : 1][13][WAVE];   // what other super-chunks contribute, parked per wave
     __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? BWD_SMAX : 1][2][STAGED ? L : 1][WAVE];
 
     const int lane = threadIdx.x & (WAVE - 1);
@@ -155,6 +156,84 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         const int cc = cok ? c0 : 0;                         // in-range column for the auxiliary table
         auto a1 = [&](int s, int slot) -> float& { return agg1[(((size_t)b * nSC + s) * 5 + slot) * C + cc]; };
         auto a2 = [&](int s, int slot) -> float& { return agg2[(((size_t)b * nSC + s) * 8 + slot) * C + cc]; };
+
+        // Long-sequence modes: what the other super-chunks contribute depends on the auxiliary tables alone, so it is
+        // folded here, before this tile's rows are requested (the temporaries are dead by then).  Entries are fetched
+        // eight (four where the z-sums come along) per direction at a time -- one memory round trip per batch instead of one per super-chunk; the forward
+        // aggregates are summed at the running maximum of the scales met so far (integers: re-scaling is an exact
+        // ldexp) and brought to the sequence's common scale R at the end; the z-sums already are at 2^-R.
+        if (MODE >= 2) {
+            float r_seq = NEG_BIG, a_in = 0.f, b_in = 0.f, c_in = 0.f, d_in = 0.f;
+            ZScan p_in, f_in;
+            constexpr int NB = MODE == 3 ? 4 : 8;
+            const float GS = fast_exp2(-om * (float)(S * L)), nSL = (float)(S * L);
+            // uniform entry offsets go into the scalar offset of a buffer load: one address register for all of them
+            const __amdgpu_buffer_rsrc_t r1d = make_rsrc(agg1 + (size_t)b * nSC * 5 * C, (unsigned)((size_t)nSC * 5 * C * 4));
+            const __amdgpu_buffer_rsrc_t r2d = make_rsrc(agg2 + (size_t)b * nSC * 8 * C, (unsigned)((size_t)nSC * 8 * C * 4));
+            const unsigned vcol = (unsigned)cc * 4u;
+            auto g1 = [&](int s, int slot) -> float {
+                return __builtin_bit_cast(float, BufRaw<4>::ld(r1d, vcol, (unsigned)((s * 5 + slot) * C) * 4u));
+            };
+            auto g2 = [&](int s, int slot) -> float {
+                return __builtin_bit_cast(float, BufRaw<4>::ld(r2d, vcol, (unsigned)((s * 8 + slot) * C) * 4u));
+            };
+            const float r_own = g1(sc, 2);
+            float r1 = NEG_BIG, r2 = NEG_BIG;
+            const int n_before = sc, n_after = nSC - 1 - sc;
+            for (int j0 = 0; j0 < n_before || j0 < n_after; j0 += NB) {
+                float pr[NB], p0[NB], p1[NB], fr[NB], f0[NB], f1[NB], pz[NB][4], fz[NB][4];
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {                           // all conditions are workgroup-uniform
+                    const int sp = j0 + i, sf = nSC - 1 - j0 - i;
+                    if (j0 + i < n_before) {
+                        pr[i] = g1(sp, 2); p0[i] = g1(sp, 0); p1[i] = g1(sp, 1);
+                        if (MODE == 3) {
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) pz[i][x] = g2(sp, x);
+                        }
+                    }
+                    if (j0 + i < n_after) {
+                        fr[i] = g1(sf, 2); f0[i] = g1(sf, 3); f1[i] = g1(sf, 4);
+                        if (MODE == 3) {
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) fz[i][x] = g2(sf, 4 + x);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    if (j0 + i < n_before) {
+                        const float m = fmaxf(r1, pr[i]);
+                        const int so = shift_of(r1 - m), sn = shift_of(pr[i] - m);
+                        a_in = fmaf(GS, ldexpf(a_in, so), ldexpf(p0[i], sn));
+                        b_in = fmaf(GS, ldexpf(b_in, so), ldexpf(p1[i], sn));
+                        r1 = m;
+                        if (MODE == 3) p_in.hop(GS, nSL, pz[i][0], pz[i][1], pz[i][2], pz[i][3]);
+                    }
+                    if (j0 + i < n_after) {
+                        const float m = fmaxf(r2, fr[i]);
+                        const int so = shift_of(r2 - m), sn = shift_of(fr[i] - m);
+                        c_in = fmaf(GS, ldexpf(c_in, so), ldexpf(f0[i], sn));
+                        d_in = fmaf(GS, ldexpf(d_in, so), ldexpf(f1[i], sn));
+                        r2 = m;
+                        if (MODE == 3) f_in.hop(GS, nSL, fz[i][0], fz[i][1], fz[i][2], fz[i][3]);
+                    }
+                }
+            }
+            r_seq = fmaxf(r_own, fmaxf(r1, r2));                         // common scale of the whole sequence
+            const int s1 = shift_of(r1 - r_seq), s2 = shift_of(r2 - r_seq);
+            // parked in this wave's own LDS slots until they are needed after the exchange: thirteen registers less
+            // across the forward pass, where the kernel has none to spare
+            float (*in)[WAVE] = s_in[wave];
+            in[0][lane] = ldexpf(a_in, s1); in[1][lane] = ldexpf(b_in, s1);
+            in[2][lane] = ldexpf(c_in, s2); in[3][lane] = ldexpf(d_in, s2);
+            in[4][lane] = r_seq;
+            if (MODE == 3) {
+                in[5][lane] = p_in.s0; in[6][lane] = p_in.s1; in[7][lane] = p_in.l0; in[8][lane] = p_in.l1;
+                in[9][lane] = f_in.s0; in[10][lane] = f_in.s1; in[11][lane] = f_in.l0; in[12][lane] = f_in.l1;
+            }
+            asm volatile("" ::: "memory");                               // the row loads below stay below
+        }
 
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes);
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
@@ -224,13 +303,13 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             float la[BWD_SMAX], lb[BWD_SMAX], lc[BWD_SMAX], ld[BWD_SMAX], lr[BWD_SMAX];
 #pragma unroll
             for (int s = 0; s < BWD_SMAX; ++s) {
-                const int ss = s < S ? s : S - 1;
-                la[s] = s1[ss][0][lane]; lb[s] = s1[ss][1][lane]; lr[s] = s1[ss][2][lane];
-                lc[s] = s1[ss][3][lane]; ld[s] = s1[ss][4][lane];
+                // slots of waves the workgroup does not have hold stale data: read (constant LDS offsets), never used
+                la[s] = s1[s][0][lane]; lb[s] = s1[s][1][lane]; lr[s] = s < S ? s1[s][2][lane] : NEG_BIG;
+                lc[s] = s1[s][3][lane]; ld[s] = s1[s][4][lane];
             }
             float r = NEG_BIG;
             if (MODE >= 2) {
-                for (int s = 0; s < nSC; ++s) r = fmaxf(r, a1(s, 2));       // common scale of the whole sequence
+                r = s_in[wave][4][lane];
             } else {
 #pragma unroll
                 for (int s = 0; s < BWD_SMAX; ++s) r = fmaxf(r, lr[s]);
@@ -258,19 +337,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                 wg_barrier();                                // s1 is rewritten by the next tile
                 continue;
             }
-            if (MODE >= 2) {
-                const float GS = fast_exp2(-om * (float)(S * L));
-                for (int s = 0; s < sc; ++s) {
-                    const int sh = shift_of(a1(s, 2) - r);
-                    a = fmaf(GS, a, ldexpf(a1(s, 0), sh));
-                    bb = fmaf(GS, bb, ldexpf(a1(s, 1), sh));
-                }
-                for (int s = nSC - 1; s > sc; --s) {
-                    const int sh = shift_of(a1(s, 2) - r);
-                    c = fmaf(GS, c, ldexpf(a1(s, 3), sh));
-                    d = fmaf(GS, d, ldexpf(a1(s, 4), sh));
-                }
-            }
+            if (MODE >= 2) { a = s_in[wave][0][lane]; bb = s_in[wave][1][lane]; c = s_in[wave][2][lane]; d = s_in[wave][3][lane]; }
 #pragma unroll
             for (int s = 0; s < BWD_SMAX; ++s)
                 if (s < wave) {
@@ -360,9 +427,9 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             const float nL = (float)L;
             if (MODE == 3) {
                 // the other super-chunks (their sums are at the common scale 2^-R), nearest last; then to my scale
-                const float GS = fast_exp2(-om * (float)(S * L)), nSL = (float)(S * L);
-                for (int s = 0; s < sc; ++s) p.hop(GS, nSL, a2(s, 0), a2(s, 1), a2(s, 2), a2(s, 3));
-                for (int s = nSC - 1; s > sc; --s) f.hop(GS, nSL, a2(s, 4), a2(s, 5), a2(s, 6), a2(s, 7));
+                const float (*in)[WAVE] = s_in[wave];
+                p.s0 = in[5][lane]; p.s1 = in[6][lane]; p.l0 = in[7][lane]; p.l1 = in[8][lane];
+                f.s0 = in[9][lane]; f.s1 = in[10][lane]; f.l0 = in[11][lane]; f.l1 = in[12][lane];
                 const int sh = shift_of(-Rw_to_R);                        // 2^(Rw - R) <= 1
                 p.s0 = ldexpf(p.s0, sh); p.s1 = ldexpf(p.s1, sh); p.l0 = ldexpf(p.l0, sh); p.l1 = ldexpf(p.l1, sh);
                 f.s0 = ldexpf(f.s0, sh); f.s1 = ldexpf(f.s1, sh); f.l0 = ldexpf(f.l0, sh); f.l1 = ldexpf(f.l1, sh);
@@ -392,13 +459,16 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         }
         const __amdgpu_buffer_rsrc_t rgk = make_rsrc(gk_ + slab, bytes);
         const __amdgpu_buffer_rsrc_t rgv = make_rsrc(gv_ + slab, bytes);
+        // the per-token offsets are formed again here (one add each) instead of staying in 28 registers since the loads
+        unsigned vst = voff0;
+        asm volatile("" : "+v"(vst));
 #pragma unroll
         for (int j = L - 1; j >= 0; --j) {
             const float gv = E[j] * (GV[j] + f.s0);
             const float gk = fmaf(V[j], gv, -E[j] * (GK[j] + f.s1));
             gw_acc = fmaf(-E[j], fmaf(V[j], f.l0, -f.l1), gw_acc);
             f.push(gd, Z[j], ZY[j]);
-            const unsigned vo = voff0 + (unsigned)j * row;    // tokens >= T fall outside the descriptor
+            const unsigned vo = vst + (unsigned)j * row;      // tokens >= T fall outside the descriptor
             store1<IO>(rgv, vo, gv);
             store1<IO>(rgk, vo, gk);
         }

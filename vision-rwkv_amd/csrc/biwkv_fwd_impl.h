@@ -278,8 +278,8 @@ struct BiwkvTile {
                         float tr[NB], t0[NB], t1[NB];
 #pragma unroll
                         for (int i = 0; i < NB; ++i) {
-                            const int se = s0 + i < q.sc ? s0 + i : q.sc - 1;          // wave-uniform
-                            tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 0, e); t1[i] = ws_at(se, 1, e);
+                            const int se = s0 + i;                                     // wave-uniform
+                            if (se < q.sc) { tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 0, e); t1[i] = ws_at(se, 1, e); }
                         }
 #pragma unroll
                         for (int i = 0; i < NB; ++i)
@@ -295,8 +295,8 @@ struct BiwkvTile {
                         float tr[NB], t0[NB], t1[NB];
 #pragma unroll
                         for (int i = 0; i < NB; ++i) {
-                            const int se = s0 - i > q.sc ? s0 - i : q.sc + 1;
-                            tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 3, e); t1[i] = ws_at(se, 4, e);
+                            const int se = s0 - i;
+                            if (se > q.sc) { tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 3, e); t1[i] = ws_at(se, 4, e); }
                         }
 #pragma unroll
                         for (int i = 0; i < NB; ++i)
