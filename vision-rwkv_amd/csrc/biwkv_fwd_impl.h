@@ -318,12 +318,20 @@ struct BiwkvTile {
             // this tile's rows have landed (loads and the previous tile's stores share one counter and may
             // retire in either order, so the wait is for all of them)
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (q.tw + L <= T) {                         // wave-uniform: every token of the chunk exists
 #pragma unroll
-            for (int j = 0; j < L; ++j) {
-                const bool tok = q.tw + j < T;
-                const float kk = to_f32(s_stage[j * WAVE + lane]), vv = to_f32(s_stage[(LR + j) * WAVE + lane]);
-                X0[j][0] = tok ? kk : NEG_INF;
-                X1[j][0] = tok ? vv : 0.f;               // rows past T were not written: LDS holds stale bits
+                for (int j = 0; j < L; ++j) {
+                    X0[j][0] = to_f32(s_stage[j * WAVE + lane]);
+                    X1[j][0] = to_f32(s_stage[(LR + j) * WAVE + lane]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < L; ++j) {
+                    const bool tok = q.tw + j < T;
+                    const float kk = to_f32(s_stage[j * WAVE + lane]), vv = to_f32(s_stage[(LR + j) * WAVE + lane]);
+                    X0[j][0] = tok ? kk : NEG_INF;
+                    X1[j][0] = tok ? vv : 0.f;           // rows past T were not written: LDS holds stale bits
+                }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
             if (next < g.n_tiles) issue_stage(next, wun);
