@@ -139,3 +139,40 @@ def test_vrwkv6_backbone_fused_equals_eager_and_trains(cls):
         g = getattr(net.layers[0].att, name).grad
         assert g is not None and torch.isfinite(g).all(), name
     assert net.layers[0].att.time_faaaa.grad.abs().sum().item() > 0
+
+
+@pytest.mark.parametrize("kind", ["vrwkv", "vrwkv6"])
+def test_reference_checkpoint_keys_load(kind):
+    """CPU: a state dict with the reference's key names (vrwkv.py:351-358 keeps the patch embedding as
+    `patch_embed.projection.*`; whole-model checkpoints prefix `backbone.` and carry a head) loads into the
+    backbone, including a position table trained on another grid."""
+    import vision_rwkv_amd as ops
+    torch.manual_seed(0)
+    if kind == "vrwkv":
+        mk = lambda img: ops.VRWKV(img_size=img, patch_size=16, embed_dims=64, depth=2, init_values=1e-5,
+                                   post_norm=True, key_norm=True)
+        expect = {"layers.0.att.spatial_decay", "layers.0.att.spatial_first", "layers.0.att.spatial_mix_k",
+                  "layers.0.att.spatial_mix_v", "layers.0.att.spatial_mix_r", "layers.1.ffn.spatial_mix_k",
+                  "layers.0.gamma1", "layers.0.ln0.weight", "layers.1.att.key_norm.weight", "ln1.weight", "pos_embed"}
+    else:
+        mk = lambda img: ops.VRWKV6(img_size=img, patch_size=16, embed_dims=128, depth=2, num_heads=2)
+        expect = {"layers.0.att.time_maa_x", "layers.0.att.time_maa_w1", "layers.0.att.time_decay",
+                  "layers.0.att.time_decay_w2", "layers.0.att.time_faaaa", "layers.0.att.ln_x.weight",
+                  "layers.0.att.gate.weight", "layers.1.ffn.spatial_mix_r", "ln1.weight", "pos_embed"}
+    src = mk(48)                                   # "pre-trained" on a 3x3 grid
+    for p in src.parameters():
+        torch.nn.init.normal_(p)
+    own = src.state_dict()
+    assert expect <= set(own)
+    ckpt = {"state_dict": {"backbone." + k.replace("patch_embed.", "patch_embed.projection."): v.clone()
+                           for k, v in own.items()}}
+    ckpt["state_dict"]["head.fc.weight"] = torch.zeros(10, 64)
+    dst = mk(32)                                   # built for a 2x2 grid
+    res = dst.load_reference_state_dict(ckpt)
+    assert not res.missing_keys and not res.unexpected_keys
+    assert dst.patch_resolution == (3, 3)
+    for k, v in dst.state_dict().items():
+        assert torch.equal(v, own[k]), k
+    bad = {"backbone.layers.0.att.no_such_parameter": torch.zeros(1)}
+    with pytest.raises(KeyError):
+        mk(32).load_reference_state_dict(bad)

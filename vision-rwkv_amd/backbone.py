@@ -146,6 +146,35 @@ class VRWKV(nn.Module):
         if final_norm:
             self.ln1 = nn.LayerNorm(embed_dims)
 
+    def load_reference_state_dict(self, state_dict, strict=True):
+        """Load a checkpoint written by the reference backbones (vrwkv.py:322-432, vrwkv6.py, the mmdet / mmseg /
+        classification_internimage copies).  Their parameter names are the ones used here except for the patch
+        embedding, which mmcv's PatchEmbed keeps as `patch_embed.projection.{weight,bias}` (vrwkv.py:351-358);
+        whole-model checkpoints carry a `backbone.` prefix and other modules' entries (`head.*`, `neck.*`), which are
+        dropped.  A position table trained on another grid replaces this model's table and pre-training grid (it is
+        interpolated to the input's grid in forward, as vrwkv.py:411-415 does).  Returns what
+        nn.Module.load_state_dict returns."""
+        sd = state_dict.get("state_dict", state_dict)
+        if any(k.startswith("backbone.") for k in sd):
+            sd = {k[len("backbone."):]: v for k, v in sd.items() if k.startswith("backbone.")}
+        own = set(self.state_dict().keys())
+        out = {}
+        for k, v in sd.items():
+            k = k.replace("patch_embed.projection.", "patch_embed.")
+            if k in own:
+                out[k] = v
+            elif strict and k.split(".")[0] in {"patch_embed", "pos_embed", "layers", "ln1", "cls_token"}:
+                raise KeyError(f"unexpected backbone entry {k!r} in the checkpoint")
+        pe = out.get("pos_embed")
+        if pe is not None and pe.shape != self.pos_embed.shape:
+            n = pe.shape[1]
+            side = int(round(n ** 0.5))
+            if pe.dim() != 3 or pe.shape[2] != self.pos_embed.shape[2] or side * side != n:
+                raise RuntimeError(f"pos_embed of shape {tuple(pe.shape)} does not fit this model")
+            self.pos_embed = nn.Parameter(torch.zeros_like(pe, dtype=self.pos_embed.dtype, device=self.pos_embed.device))
+            self.patch_resolution = (side, side)
+        return self.load_state_dict(out, strict=strict)
+
     def _pos_embed_for(self, res):
         """Position embedding at grid `res`; in eval mode the interpolated table is computed once per grid
         (the reference re-runs the bicubic resize in every forward, vrwkv.py:411-415)."""
