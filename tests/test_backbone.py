@@ -176,3 +176,19 @@ def test_reference_checkpoint_keys_load(kind):
     bad = {"backbone.layers.0.att.no_such_parameter": torch.zeros(1)}
     with pytest.raises(KeyError):
         mk(32).load_reference_state_dict(bad)
+
+
+def test_pos_embed_resize_restates_the_interpolation():
+    """CPU: resize_pos_embed against a direct F.interpolate of the grid part (embed.py:6-47), with and without
+    extra tokens, and the identity when the grids agree."""
+    from vision_rwkv_amd.backbone import resize_pos_embed
+    import torch.nn.functional as F
+    torch.manual_seed(1)
+    pe = torch.randn(1, 1 + 12, 8)
+    out = resize_pos_embed(pe, (3, 4), (6, 5), "bicubic", num_extra_tokens=1)
+    grid = pe[:, 1:].reshape(1, 3, 4, 8).permute(0, 3, 1, 2)
+    ref = F.interpolate(grid, size=(6, 5), mode="bicubic", align_corners=False).flatten(2).transpose(1, 2)
+    assert out.shape == (1, 31, 8) and torch.equal(out[:, :1], pe[:, :1]) and torch.allclose(out[:, 1:], ref)
+    assert resize_pos_embed(pe[:, 1:], (3, 4), (3, 4)) is not None and resize_pos_embed(pe[:, 1:], (3, 4), (3, 4)).shape == (1, 12, 8)
+    with pytest.raises(RuntimeError):
+        resize_pos_embed(pe, (3, 4), (6, 5))

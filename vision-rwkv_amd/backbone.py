@@ -17,13 +17,20 @@ import torch.nn.functional as F
 from .ops import RUN_CUDA, q_shift, q_shift_mix
 
 
-def resize_pos_embed(pos_embed, src_shape, dst_shape, mode="bicubic"):
+def resize_pos_embed(pos_embed, src_shape, dst_shape, mode="bicubic", num_extra_tokens=0):
+    """Position table (1, extra + Hs*Ws, C) resampled to the grid dst_shape, extra tokens passed through: the
+    interpolation of detection/mmdet_custom/models/utils/embed.py:6-47 (F.interpolate, align_corners=False), which
+    the backbones call with no extra tokens (vrwkv.py:411-415)."""
     if tuple(src_shape) == tuple(dst_shape):
         return pos_embed
     _, L, C = pos_embed.shape
-    w = pos_embed.reshape(1, src_shape[0], src_shape[1], C).permute(0, 3, 1, 2)
+    if L != src_shape[0] * src_shape[1] + num_extra_tokens:
+        raise RuntimeError(f"pos_embed has {L} tokens, expected {src_shape[0]}*{src_shape[1]}+{num_extra_tokens}")
+    extra, grid = pos_embed[:, :num_extra_tokens], pos_embed[:, num_extra_tokens:]
+    w = grid.reshape(1, src_shape[0], src_shape[1], C).permute(0, 3, 1, 2)
     w = F.interpolate(w.float(), size=dst_shape, align_corners=False, mode=mode).to(pos_embed.dtype)
-    return torch.flatten(w, 2).transpose(1, 2)
+    w = torch.flatten(w, 2).transpose(1, 2)
+    return torch.cat((extra, w), dim=1) if num_extra_tokens else w
 
 
 def _mix(x, mixes, shift_pixel, gamma, patch_resolution, fused):
