@@ -200,6 +200,9 @@ def backbone_section(torch, ops, steps, warmup):
             if hasattr(m, "fused_shift"):
                 m.fused_shift = False
         ms_fwd_eager_shift = timed(lambda: net(img), steps, warmup)
+        ops.ops.ROW_FUSE_ENABLED = False
+        ms_fwd_unfused = timed(lambda: net(img), steps, warmup)
+        ops.ops.ROW_FUSE_ENABLED = True
         Tn, Cn = (S // 16) ** 2, 1024
         att = net.layers[0].att
         k = torch.randn(Bn, Tn, Cn, device=dev, dtype=torch.bfloat16)
@@ -218,6 +221,7 @@ def backbone_section(torch, ops, steps, warmup):
     return {"workload": f"VRWKV-L forward, batch {Bn}, {S}x{S}, T={Tn}, C={Cn}, 24 blocks, bf16, random weights",
             "ms_per_forward": round(ms_fwd, 3), "images_per_s": round(Bn / ms_fwd * 1e3, 1),
             "ms_per_forward_unfused_shift": round(ms_fwd_eager_shift, 3),
+            "ms_per_forward_all_elementwise_in_pytorch": round(ms_fwd_unfused, 3),
             "biwkv_ms_per_forward": round(ms_wkv, 3), "biwkv_share": round(ms_wkv / ms_fwd, 4),
             "vrwkv6_b": {"workload": "VRWKV6-B forward, batch 64, 224x224, T=196, C=768, 12 heads, 12 blocks, bf16, "
                                      "random weights",

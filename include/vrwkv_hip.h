@@ -105,6 +105,18 @@ int vrwkv_qshift_mix(const void* x, const float* mix, void* const* out, int n_mi
                      int B, int T, int C, int Hp, int Wp, int shift_pixel, int quarter_width,
                      int head_dim, int io_dtype, void* hip_stream);
 
+/* ---- fused row-wise epilogues of the blocks (the elementwise steps behind the operator and the GEMMs) ----
+ * For every row of N channels:  y = LayerNorm(pre(a)) (weight, bias; LayerNorm skipped when ln_weight is NULL),
+ * out = y (post 0) | sigmoid(other) * y (post 1) | other + gamma * y (post 2, gamma NULL = 1); pre 0 = identity,
+ * pre 1 = relu(a)^2.  Replaces, in one pass over memory, the PyTorch-op sequences of
+ * classification/mmcls_custom/models/backbones/vrwkv.py:184-186 (key_norm, sr * rwkv), :256-261 (relu^2, key_norm,
+ * sigmoid gate) and :300-313 (residual with layer scale, post- or pre-norm).  The reference has no native code here.
+ * a, other, out: (rows, N) of io_dtype; ln_weight, ln_bias, gamma: (N,) of io_dtype; all 16-byte aligned;
+ * N a multiple of the 4 (fp32) or 8 (16-bit) elements in 16 bytes and at most 1024 such vectors. */
+int vrwkv_rowfuse(const void* a, const void* other, const void* ln_weight, const void* ln_bias,
+                  const void* gamma, void* out, long long rows, int N, int pre, int post, float eps,
+                  int io_dtype, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

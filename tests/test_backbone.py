@@ -192,3 +192,37 @@ def test_pos_embed_resize_restates_the_interpolation():
     assert resize_pos_embed(pe[:, 1:], (3, 4), (3, 4)) is not None and resize_pos_embed(pe[:, 1:], (3, 4), (3, 4)).shape == (1, 12, 8)
     with pytest.raises(RuntimeError):
         resize_pos_embed(pe, (3, 4), (6, 5))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,dtype", [(1024, torch.bfloat16), (4096, torch.bfloat16), (768, torch.float32),
+                                     (3072, torch.float32), (64, torch.float16), (8192, torch.bfloat16)])
+def test_row_fuse_against_tensor_ops(N, dtype):
+    """The fused row epilogues against the PyTorch-op sequence evaluated in fp32 on the same (rounded) inputs:
+    every pre / LayerNorm / post combination the blocks use, rows that do not fill a workgroup.
+    Tolerance: 2e-3 of the row scale for fp32 I/O (fast exp / rcp in the gate), one 16-bit rounding otherwise."""
+    import vision_rwkv_amd as ops
+    dev = "cuda:0"
+    torch.manual_seed(N)
+    rows = (3, 7)                                   # 21 rows: the last workgroup is partial
+    a = torch.randn(*rows, N, device=dev).to(dtype)
+    o = torch.randn(*rows, N, device=dev).to(dtype)
+    w, b, g = (torch.randn(N, device=dev).to(dtype) for _ in range(3))
+    combos = [(ops.ops.PRE_NONE, ops.ops.POST_SIGMOID_GATE, True), (ops.ops.PRE_NONE, ops.ops.POST_SIGMOID_GATE, False),
+              (ops.ops.PRE_RELU_SQ, ops.ops.POST_NONE, True), (ops.ops.PRE_RELU_SQ, ops.ops.POST_NONE, False),
+              (ops.ops.PRE_NONE, ops.ops.POST_RESIDUAL, True), (ops.ops.PRE_NONE, ops.ops.POST_RESIDUAL, False),
+              (ops.ops.PRE_NONE, ops.ops.POST_NONE, True)]
+    tol = 2e-3 if dtype == torch.float32 else 1e-2
+    for pre, post, ln in combos:
+        for gamma in ((g, None) if post == ops.ops.POST_RESIDUAL else (None,)):
+            with torch.no_grad():
+                got = ops.row_fuse(a, o if post else None, w if ln else None, b if ln else None, gamma, pre, post)
+            f = lambda t: t.float() if t is not None else None
+            ref = ops.row_fuse_tensor_ops(f(a), f(o), f(w) if ln else None, f(b) if ln else None, f(gamma), pre, post)
+            assert got.dtype == dtype and got.shape == a.shape
+            err = (got.float() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-6)
+            assert err <= tol, (pre, post, ln, gamma is not None, err)
+    # a gradient is wanted: the tensor ops run and autograd works
+    a2 = a.float().requires_grad_(True)
+    ops.row_fuse(a2, o.float(), w.float(), b.float(), g.float(), ops.ops.PRE_NONE, ops.ops.POST_RESIDUAL).sum().backward()
+    assert a2.grad is not None and torch.isfinite(a2.grad).all()

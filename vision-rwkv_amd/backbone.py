@@ -14,7 +14,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .ops import RUN_CUDA, q_shift, q_shift_mix
+from .ops import (RUN_CUDA, q_shift, q_shift_mix, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE, POST_SIGMOID_GATE,
+                  POST_RESIDUAL)
 
 
 def resize_pos_embed(pos_embed, src_shape, dst_shape, mode="bicubic", num_extra_tokens=0):
@@ -69,13 +70,14 @@ class VRWKV_SpatialMix(nn.Module):
                               self.channel_gamma, patch_resolution, self.fused_shift)
         else:
             xk = xv = xr = x
-        k, v = self.key(xk), self.value(xv)
-        sr = torch.sigmoid(self.receptance(xr))
+        k, v, r = self.key(xk), self.value(xv), self.receptance(xr)
         y = RUN_CUDA(self.spatial_decay / T, self.spatial_first / T, k, v)      # vrwkv.py:183
-        y = y.to(sr.dtype)
-        if self.key_norm is not None:
-            y = self.key_norm(y)
-        return self.output(sr * y)
+        y = y.to(r.dtype)
+        # key_norm and the sigmoid gate (vrwkv.py:184-186) in one pass; tensor ops under autograd
+        kn = self.key_norm
+        y = row_fuse(y, r, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
+                     PRE_NONE, POST_SIGMOID_GATE, kn.eps if kn is not None else 1e-5)
+        return self.output(y)
 
 
 class VRWKV_ChannelMix(nn.Module):
@@ -99,10 +101,11 @@ class VRWKV_ChannelMix(nn.Module):
                           patch_resolution, self.fused_shift)
         else:
             xk = xr = x
-        k = torch.square(torch.relu(self.key(xk)))
-        if self.key_norm is not None:
-            k = self.key_norm(k)
-        return torch.sigmoid(self.receptance(xr)) * self.value(k)
+        # relu^2 (+ key_norm) and the sigmoid gate (vrwkv.py:256-261), one pass each; tensor ops under autograd
+        kn = self.key_norm
+        k = row_fuse(self.key(xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
+                     PRE_RELU_SQ, POST_NONE, kn.eps if kn is not None else 1e-5)
+        return row_fuse(self.value(k), self.receptance(xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
 
 
 class Block(nn.Module):
@@ -123,14 +126,16 @@ class Block(nn.Module):
     def forward(self, x, patch_resolution):
         if self.layer_id == 0:
             x = self.ln0(x)
-        g1 = self.gamma1 if self.layer_scale else 1.0
-        g2 = self.gamma2 if self.layer_scale else 1.0
-        if self.post_norm:                                   # vrwkv.py:300-306
-            x = x + g1 * self.ln1(self.att(x, patch_resolution))
-            x = x + g2 * self.ln2(self.ffn(x, patch_resolution))
+        g1 = self.gamma1 if self.layer_scale else None
+        g2 = self.gamma2 if self.layer_scale else None
+        # residual with layer scale (vrwkv.py:300-313): x + gamma * ln(branch(x)) or x + gamma * branch(ln(x)), the
+        # scale, the add and the post-norm in one pass; tensor ops under autograd
+        if self.post_norm:
+            x = row_fuse(self.att(x, patch_resolution), x, self.ln1.weight, self.ln1.bias, g1, PRE_NONE, POST_RESIDUAL, self.ln1.eps)
+            x = row_fuse(self.ffn(x, patch_resolution), x, self.ln2.weight, self.ln2.bias, g2, PRE_NONE, POST_RESIDUAL, self.ln2.eps)
         else:
-            x = x + g1 * self.att(self.ln1(x), patch_resolution)
-            x = x + g2 * self.ffn(self.ln2(x), patch_resolution)
+            x = row_fuse(self.att(self.ln1(x), patch_resolution), x, None, None, g1, PRE_NONE, POST_RESIDUAL)
+            x = row_fuse(self.ffn(self.ln2(x), patch_resolution), x, None, None, g2, PRE_NONE, POST_RESIDUAL)
         return x
 
 

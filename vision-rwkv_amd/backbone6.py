@@ -11,7 +11,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .backbone import VRWKV
-from .ops import HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix
+from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE,
+                  POST_SIGMOID_GATE, POST_RESIDUAL)
 
 
 def q_shift_multihead(x, shift_pixel=1, head_dim=HEAD_SIZE, patch_resolution=None, with_cls_token=False):
@@ -110,10 +111,10 @@ class VRWKV_ChannelMix_V6(nn.Module):
     def forward(self, x, patch_resolution):
         xk, xr = _shift_and_mix(x, [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel, patch_resolution,
                                 self.with_cls_token, self.fused_shift)
-        k = torch.square(torch.relu(self.key(xk)))
-        if self.key_norm is not None:
-            k = self.key_norm(k)
-        return torch.sigmoid(self.receptance(xr)) * self.value(k)
+        kn = self.key_norm                                   # relu^2 (+ key_norm), then the sigmoid gate: one pass each
+        k = row_fuse(self.key(xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
+                     PRE_RELU_SQ, POST_NONE, kn.eps if kn is not None else 1e-5)
+        return row_fuse(self.value(k), self.receptance(xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
 
 
 class Block6(nn.Module):
@@ -135,14 +136,14 @@ class Block6(nn.Module):
     def forward(self, x, patch_resolution):
         if self.layer_id == 0:
             x = self.ln0(x)
-        g1 = self.gamma1 if self.layer_scale else 1.0
-        g2 = self.gamma2 if self.layer_scale else 1.0
-        if self.post_norm:
-            x = x + g1 * self.ln1(self.att(x, patch_resolution))
-            x = x + g2 * self.ln2(self.ffn(x, patch_resolution))
+        g1 = self.gamma1 if self.layer_scale else None
+        g2 = self.gamma2 if self.layer_scale else None
+        if self.post_norm:                                   # scale, add and post-norm in one pass
+            x = row_fuse(self.att(x, patch_resolution), x, self.ln1.weight, self.ln1.bias, g1, PRE_NONE, POST_RESIDUAL, self.ln1.eps)
+            x = row_fuse(self.ffn(x, patch_resolution), x, self.ln2.weight, self.ln2.bias, g2, PRE_NONE, POST_RESIDUAL, self.ln2.eps)
         else:
-            x = x + g1 * self.att(self.ln1(x), patch_resolution)
-            x = x + g2 * self.ffn(self.ln2(x), patch_resolution)
+            x = row_fuse(self.att(self.ln1(x), patch_resolution), x, None, None, g1, PRE_NONE, POST_RESIDUAL)
+            x = row_fuse(self.ffn(self.ln2(x), patch_resolution), x, None, None, g2, PRE_NONE, POST_RESIDUAL)
         return x
 
 

@@ -278,3 +278,47 @@ def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, hea
         _lib.check(_lib.lib().vrwkv_qshift_mix(x.data_ptr(), mix.data_ptr(), ptrs, len(outs), B, T, C, Hp, Wp,
                                                shift_pixel, g, head_dim, _DT[x.dtype], _stream_ptr(x.device)))
     return outs
+
+
+PRE_NONE, PRE_RELU_SQ = 0, 1
+POST_NONE, POST_SIGMOID_GATE, POST_RESIDUAL = 0, 1, 2
+ROW_FUSE_ENABLED = True      # set False to make row_fuse run the tensor-op sequence everywhere (for comparisons)
+
+
+def row_fuse_tensor_ops(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NONE, post=POST_NONE, eps=1e-5):
+    """The PyTorch-op sequence row_fuse replaces (what the reference runs: vrwkv.py:184-186, :256-261, :300-313);
+    used under autograd and wherever the kernel does not apply."""
+    y = torch.square(torch.relu(a)) if pre == PRE_RELU_SQ else a
+    if ln_weight is not None:
+        y = torch.nn.functional.layer_norm(y, (y.shape[-1],), ln_weight, ln_bias, eps)
+    if post == POST_SIGMOID_GATE:
+        y = torch.sigmoid(other) * y
+    elif post == POST_RESIDUAL:
+        y = other + (gamma * y if gamma is not None else y)
+    return y
+
+
+def row_fuse(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NONE, post=POST_NONE, eps=1e-5):
+    """One HIP kernel per row-wise epilogue of a block: out = post(LayerNorm(pre(a))) with pre = identity / relu^2,
+    LayerNorm optional, post = identity / sigmoid(other) * y / other + gamma * y.  Forward only: when a gradient is
+    needed, the tensors are not on the GPU, or the row length does not fit, the tensor ops are used instead."""
+    tensors = [t for t in (a, other, ln_weight, ln_bias, gamma) if t is not None]
+    N = a.shape[-1]
+    vec = 4 if a.dtype == torch.float32 else 8
+    fits = (ROW_FUSE_ENABLED and a.is_cuda and a.dtype in _DT and N % vec == 0 and N // vec <= 1024 and a.numel() > 0
+            and (other is None or (other.shape == a.shape and other.dtype == a.dtype))
+            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
+    if not fits:
+        return row_fuse_tensor_ops(a, other, ln_weight, ln_bias, gamma, pre, post, eps)
+    a = a.contiguous()
+    other = other.contiguous() if other is not None else None
+    par = [p.detach().reshape(-1).to(a.dtype).contiguous() if p is not None else None for p in (ln_weight, ln_bias, gamma)]
+    for p in par:
+        if p is not None and p.numel() != N:
+            raise RuntimeError("LayerNorm weight, bias and gamma must have one element per channel")
+    out = torch.empty_like(a)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().vrwkv_rowfuse(a.data_ptr(), ptr(other), ptr(par[0]), ptr(par[1]), ptr(par[2]), out.data_ptr(),
+                                            a.numel() // N, N, pre, post, float(eps), _DT[a.dtype], _stream_ptr(a.device)))
+    return out
