@@ -14,7 +14,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .ops import (RUN_CUDA, q_shift, q_shift_mix, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE, POST_SIGMOID_GATE,
+from .ops import (RUN_CUDA, bi_wkv_forward, q_shift, q_shift_mix, stack_mixes, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE, POST_SIGMOID_GATE,
                   POST_RESIDUAL)
 
 
@@ -34,10 +34,23 @@ def resize_pos_embed(pos_embed, src_shape, dst_shape, mode="bicubic", num_extra_
     return torch.cat((extra, w), dim=1) if num_extra_tokens else w
 
 
-def _mix(x, mixes, shift_pixel, gamma, patch_resolution, fused):
+def eval_cached(module, name, params, extra, make):
+    """Value derived from parameters (a dtype conversion, a stacked table), kept on the module between forward passes
+    without autograd and rebuilt when a parameter was written to (its version counter), moved or cast."""
+    key = (extra,) + tuple((p._version, p.dtype, p.device, p.data_ptr()) for p in params)
+    slot = module.__dict__.setdefault("_eval_cache", {})
+    hit = slot.get(name)
+    if hit is None or hit[0] != key:
+        hit = (key, make())
+        slot[name] = hit
+    return hit[1]
+
+
+def _mix(module, x, mixes, shift_pixel, gamma, patch_resolution, fused, head_dim=0):
     """[x*m + q_shift(x)*(1-m) for m in mixes]: one fused kernel at inference, tensor ops under autograd."""
     if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or mixes[0].requires_grad)):
-        return q_shift_mix(x.contiguous(), mixes, shift_pixel, gamma, patch_resolution)
+        table = eval_cached(module, "mix_table", mixes, x.device, lambda: stack_mixes(mixes, x.device))
+        return q_shift_mix(x.contiguous(), mixes, shift_pixel, gamma, patch_resolution, head_dim, mix_table=table)
     xx = q_shift(x, shift_pixel, gamma, patch_resolution)
     return [x * m + xx * (1 - m) for m in mixes]
 
@@ -66,12 +79,20 @@ class VRWKV_SpatialMix(nn.Module):
     def forward(self, x, patch_resolution):
         B, T, C = x.shape
         if self.shift_pixel > 0:
-            xk, xv, xr = _mix(x, [self.spatial_mix_k, self.spatial_mix_v, self.spatial_mix_r], self.shift_pixel,
+            xk, xv, xr = _mix(self, x, [self.spatial_mix_k, self.spatial_mix_v, self.spatial_mix_r], self.shift_pixel,
                               self.channel_gamma, patch_resolution, self.fused_shift)
         else:
             xk = xv = xr = x
         k, v, r = self.key(xk), self.value(xv), self.receptance(xr)
-        y = RUN_CUDA(self.spatial_decay / T, self.spatial_first / T, k, v)      # vrwkv.py:183
+        wd = self.spatial_decay.dtype
+        if torch.is_grad_enabled() or k.dtype != (wd if wd in (torch.half, torch.bfloat16) else torch.float32):
+            y = RUN_CUDA(self.spatial_decay / T, self.spatial_first / T, k, v)  # vrwkv.py:183
+        else:
+            # what WKV.forward does with these arguments, the scaled fp32 copies of w and u kept between calls
+            w, u = eval_cached(self, "wu", (self.spatial_decay, self.spatial_first), T,
+                               lambda: ((self.spatial_decay / T).float().contiguous(),
+                                        (self.spatial_first / T).float().contiguous()))
+            y = bi_wkv_forward(w, u, k.contiguous(), v.contiguous())
         y = y.to(r.dtype)
         # key_norm and the sigmoid gate (vrwkv.py:184-186) in one pass; tensor ops under autograd
         kn = self.key_norm
@@ -97,7 +118,7 @@ class VRWKV_ChannelMix(nn.Module):
 
     def forward(self, x, patch_resolution):
         if self.shift_pixel > 0:
-            xk, xr = _mix(x, [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel, self.channel_gamma,
+            xk, xr = _mix(self, x, [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel, self.channel_gamma,
                           patch_resolution, self.fused_shift)
         else:
             xk = xr = x

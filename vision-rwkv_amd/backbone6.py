@@ -10,8 +10,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .backbone import VRWKV
-from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE,
+from .backbone import VRWKV, eval_cached
+from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, stack_mixes, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE,
                   POST_SIGMOID_GATE, POST_RESIDUAL)
 
 
@@ -27,12 +27,15 @@ def q_shift_multihead(x, shift_pixel=1, head_dim=HEAD_SIZE, patch_resolution=Non
     return torch.cat((out, x[:, -1:]), dim=1) if with_cls_token else out
 
 
-def _shift_and_mix(x, mixes, shift_pixel, patch_resolution, with_cls_token, fused):
-    """[x*m + shift(x)*(1-m) for m in mixes]; one HIP kernel at inference, tensor ops under autograd."""
-    if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or mixes[0].requires_grad)):
-        return q_shift_mix(x.contiguous(), mixes, shift_pixel, 1 / 4, patch_resolution, head_dim=HEAD_SIZE)
+def _shift_and_mix(module, x, mixes, shift_pixel, patch_resolution, with_cls_token, fused, params):
+    """[x*m + shift(x)*(1-m) for m in mixes()]; one HIP kernel at inference, tensor ops under autograd.  `mixes` is a
+    callable (the vectors may be derived from `params`); at inference its stacked fp32 table is kept on the module."""
+    if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or params[0].requires_grad)):
+        table = eval_cached(module, "mix_table", params, x.device, lambda: stack_mixes(mixes(), x.device))
+        return q_shift_mix(x.contiguous(), [None] * table.shape[0], shift_pixel, 1 / 4, patch_resolution,
+                           head_dim=HEAD_SIZE, mix_table=table)
     sx = q_shift_multihead(x, shift_pixel, HEAD_SIZE, patch_resolution, with_cls_token)
-    return [x * m + sx * (1 - m) for m in mixes]
+    return [x * m + sx * (1 - m) for m in mixes()]
 
 
 class VRWKV_SpatialMix_V6(nn.Module):
@@ -70,8 +73,9 @@ class VRWKV_SpatialMix_V6(nn.Module):
     def forward(self, x, patch_resolution):
         B, T, C = x.shape
         # shift(x) and x + (shift(x) - x) * maa_x = x*(1 - maa_x) + shift(x)*maa_x in one pass over x
-        sx, xxx = _shift_and_mix(x, [torch.zeros_like(self.time_maa_x), 1 - self.time_maa_x], self.shift_pixel,
-                                 patch_resolution, self.with_cls_token, self.fused_shift)
+        sx, xxx = _shift_and_mix(self, x, lambda: [torch.zeros_like(self.time_maa_x), 1 - self.time_maa_x],
+                                 self.shift_pixel, patch_resolution, self.with_cls_token, self.fused_shift,
+                                 (self.time_maa_x,))
         xx = sx - x
         lo = torch.tanh(xxx @ self.time_maa_w1).view(B * T, 5, -1).transpose(0, 1)
         mw, mk, mv, mr, mg = torch.bmm(lo, self.time_maa_w2).view(5, B, T, C).unbind(0)
@@ -109,8 +113,9 @@ class VRWKV_ChannelMix_V6(nn.Module):
         self.value = nn.Linear(hidden, n_embd, bias=False)
 
     def forward(self, x, patch_resolution):
-        xk, xr = _shift_and_mix(x, [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel, patch_resolution,
-                                self.with_cls_token, self.fused_shift)
+        xk, xr = _shift_and_mix(self, x, lambda: [self.spatial_mix_k, self.spatial_mix_r], self.shift_pixel,
+                                patch_resolution, self.with_cls_token, self.fused_shift,
+                                (self.spatial_mix_k, self.spatial_mix_r))
         kn = self.key_norm                                   # relu^2 (+ key_norm), then the sigmoid gate: one pass each
         k = row_fuse(self.key(xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
                      PRE_RELU_SQ, POST_NONE, kn.eps if kn is not None else 1e-5)

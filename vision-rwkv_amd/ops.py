@@ -257,7 +257,13 @@ def q_shift(input, shift_pixel=1, gamma=1 / 4, patch_resolution=None):
     return out.flatten(2).transpose(1, 2)
 
 
-def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, head_dim=0):
+def stack_mixes(mixes, device):
+    """The (n_mix, C) fp32 table q_shift_mix hands to the kernel; callers that apply the same mixes again and again
+    may build it once and pass it as `mix_table`."""
+    return torch.stack([m.detach().reshape(-1).float() for m in mixes]).contiguous().to(device)
+
+
+def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, head_dim=0, mix_table=None):
     """One HIP kernel for q_shift + the token-mix lerps: returns [x*m + q_shift(x)*(1-m) for m in mixes]
     (vrwkv.py:160-163 / :248-250).  mixes: 1..3 tensors of C elements.  head_dim=64 gives the per-head
     q_shift_multihead of vrwkv6.py:75-100 (a trailing class token is passed through).  Forward only."""
@@ -266,7 +272,9 @@ def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, hea
         raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
     B, T, C = x.shape
     Hp, Wp = patch_resolution
-    mix = torch.stack([m.reshape(-1).float() for m in mixes]).contiguous().to(x.device)
+    mix = mix_table if mix_table is not None else stack_mixes(mixes, x.device)
+    if mix.shape != (len(mixes), C) or mix.dtype != torch.float32 or not mix.is_contiguous() or mix.device != x.device:
+        raise RuntimeError("mix_table must be a contiguous float32 (n_mix, C) tensor on x's device")
     if mix.shape[1] != C:
         raise RuntimeError("every mix vector must have C elements")
     outs = [torch.empty_like(x) for _ in mixes]
