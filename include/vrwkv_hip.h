@@ -117,6 +117,20 @@ int vrwkv_rowfuse(const void* a, const void* other, const void* ln_weight, const
                   const void* gamma, void* out, long long rows, int N, int pre, int post, float eps,
                   int io_dtype, void* hip_stream);
 
+/* ---- element-wise steps of the VRWKV6 spatial mix (.../backbones/vrwkv6.py:176-212), one pass each ----
+ * vrwkv_maa_mix: the five data-dependent token mixes of jit_func (:190-194),
+ *   out[i] = x + (sx - x) * (maa[i] + m[i]),  i = w, k, v, r, g;
+ *   x, sx (the shifted x), out[i]: (rows, C) of io_dtype; m: (5, rows, C) of io_dtype (the low-rank mix of :183-186);
+ *   maa: (5, C) fp32 (time_maa_w, _k, _v, _r, _g).
+ * vrwkv_groupnorm_gate: jit_func_2 (:205-211), out = GroupNorm(y) * silu(gate) with groups of `group` consecutive
+ *   channels per row (ln_x = GroupNorm(n_head, C) on the (B*T, C) view); y: (rows, C) fp32 (as the operator returns
+ *   it) or io_dtype; gate, out: (rows, C), gn_weight, gn_bias: (C,) of io_dtype (bf16 or fp16).
+ * All tensors 16-byte aligned, C a multiple of 8 (4 for fp32 maa_mix).  The reference has no native code here. */
+int vrwkv_maa_mix(const void* x, const void* sx, const void* m, const float* maa, void* const* out,
+                  long long rows, int C, int io_dtype, void* hip_stream);
+int vrwkv_groupnorm_gate(const void* y, const void* gate, const void* gn_weight, const void* gn_bias, void* out,
+                         long long rows, int C, int group, float eps, int y_dtype, int io_dtype, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

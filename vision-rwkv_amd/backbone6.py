@@ -11,7 +11,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .backbone import VRWKV, eval_cached
-from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, stack_mixes, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE,
+from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, stack_mixes, row_fuse, maa_mix, groupnorm_gate, PRE_NONE, PRE_RELU_SQ, POST_NONE,
                   POST_SIGMOID_GATE, POST_RESIDUAL)
 
 
@@ -76,24 +76,24 @@ class VRWKV_SpatialMix_V6(nn.Module):
         sx, xxx = _shift_and_mix(self, x, lambda: [torch.zeros_like(self.time_maa_x), 1 - self.time_maa_x],
                                  self.shift_pixel, patch_resolution, self.with_cls_token, self.fused_shift,
                                  (self.time_maa_x,))
-        xx = sx - x
         lo = torch.tanh(xxx @ self.time_maa_w1).view(B * T, 5, -1).transpose(0, 1)
-        mw, mk, mv, mr, mg = torch.bmm(lo, self.time_maa_w2).view(5, B, T, C).unbind(0)
-        xw = x + xx * (self.time_maa_w + mw)
-        xk = x + xx * (self.time_maa_k + mk)
-        xv = x + xx * (self.time_maa_v + mv)
-        xr = x + xx * (self.time_maa_r + mr)
-        xg = x + xx * (self.time_maa_g + mg)
+        m = torch.bmm(lo, self.time_maa_w2).view(5, B, T, C)
+        # xw..xg = x + (sx - x) * (time_maa_* + m_*)  (vrwkv6.py:190-194): one pass at inference
+        maas = (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g)
+        table = None
+        if not torch.is_grad_enabled() and x.is_cuda:
+            table = eval_cached(self, "maa_table", maas, x.device, lambda: stack_mixes(maas, x.device))
+        xw, xk, xv, xr, xg = maa_mix(x, sx, m, maas, table)
         r, k, v = self.receptance(xr), self.key(xk), self.value(xv)
-        g = F.silu(self.gate(xg))
+        gate = self.gate(xg)
         w = self.time_decay + torch.tanh(xw @ self.time_decay_w1) @ self.time_decay_w2
         y = RUN_CUDA_RWKV6(B, T, C, self.n_head, r.contiguous(), k.contiguous(), v.contiguous(),
                            w.float().contiguous(), self.time_faaaa.float())          # vrwkv6.py:217
-        y = y.to(g.dtype)
         if self.key_norm is not None:
-            y = self.key_norm(y)
-        y = self.ln_x(y.view(B * T, C)).view(B, T, C)
-        return self.output(y * g)
+            y = self.key_norm(y.to(gate.dtype))
+        # ln_x over each head's channels, times silu(gate) (vrwkv6.py:199, 205-211): one pass at inference
+        y = groupnorm_gate(y, gate, self.ln_x.weight, self.ln_x.bias, self.ln_x.num_groups, self.ln_x.eps)
+        return self.output(y)
 
 
 class VRWKV_ChannelMix_V6(nn.Module):

@@ -330,3 +330,62 @@ def row_fuse(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NO
         _lib.check(_lib.lib().vrwkv_rowfuse(a.data_ptr(), ptr(other), ptr(par[0]), ptr(par[1]), ptr(par[2]), out.data_ptr(),
                                             a.numel() // N, N, pre, post, float(eps), _DT[a.dtype], _stream_ptr(a.device)))
     return out
+
+
+def maa_mix_tensor_ops(x, sx, m, maas):
+    """vrwkv6.py:180, 190-194 as the reference writes them: xx = sx - x; x + xx * (maa_i + m_i)."""
+    xx = sx - x
+    return [x + xx * (maa + mi) for maa, mi in zip(maas, m.unbind(0))]
+
+
+def maa_mix(x, sx, m, maas, maa_table=None):
+    """The five data-dependent token mixes of VRWKV6 (vrwkv6.py:190-194) in one HIP kernel: x, sx (the shifted x):
+    (B,T,C); m: (5,B,T,C); maas: the five (C,) vectors time_maa_w, _k, _v, _r, _g (or their stacked fp32 table).
+    Forward only: tensor ops under autograd or when the kernel does not apply."""
+    C = x.shape[-1]
+    vec = 4 if x.dtype == torch.float32 else 8
+    tensors = [x, sx, m] + list(maas)
+    fits = (ROW_FUSE_ENABLED and x.is_cuda and x.dtype in _DT and C % vec == 0 and x.numel() > 0
+            and sx.shape == x.shape and sx.dtype == x.dtype and m.dtype == x.dtype and tuple(m.shape) == (5,) + tuple(x.shape)
+            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
+    if not fits:
+        return maa_mix_tensor_ops(x, sx, m, maas)
+    x, sx, m = x.contiguous(), sx.contiguous(), m.contiguous()
+    table = maa_table if maa_table is not None else stack_mixes(maas, x.device)
+    if tuple(table.shape) != (5, C) or table.dtype != torch.float32 or not table.is_contiguous():
+        raise RuntimeError("maa table must be a contiguous float32 (5, C) tensor")
+    outs = [torch.empty_like(x) for _ in range(5)]
+    ptrs = (ctypes.c_void_p * 5)(*[o.data_ptr() for o in outs])
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().vrwkv_maa_mix(x.data_ptr(), sx.data_ptr(), m.data_ptr(), table.data_ptr(), ptrs,
+                                            x.numel() // C, C, _DT[x.dtype], _stream_ptr(x.device)))
+    return outs
+
+
+def groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
+    """vrwkv6.py:205-211 and :199: ln_x on the (B*T, C) view, times silu(gate)."""
+    C = y.shape[-1]
+    yn = torch.nn.functional.group_norm(y.to(gate.dtype).reshape(-1, C), n_groups, gn_weight, gn_bias, eps)
+    return yn.view(gate.shape) * torch.nn.functional.silu(gate)
+
+
+def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
+    """GroupNorm(n_groups, C) of every token of y (fp32 as RUN_CUDA_RWKV6 returns it, or gate's dtype) times
+    silu(gate), in one HIP kernel (vrwkv6.py:199, 205-211).  Forward only, 16-bit gate / output; tensor ops otherwise."""
+    C = y.shape[-1]
+    group = C // n_groups if n_groups > 0 and C % n_groups == 0 else 0
+    tensors = [y, gate, gn_weight, gn_bias]
+    fits = (ROW_FUSE_ENABLED and y.is_cuda and gate.dtype in (torch.bfloat16, torch.float16) and y.shape == gate.shape
+            and y.dtype in (torch.float32, gate.dtype) and group in (8, 16, 32, 64, 128) and y.numel() > 0
+            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
+    if not fits:
+        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
+    y, gate = y.contiguous(), gate.contiguous()
+    w = gn_weight.detach().to(gate.dtype).contiguous()
+    b = gn_bias.detach().to(gate.dtype).contiguous()
+    out = torch.empty_like(gate)
+    with torch.cuda.device(y.device):
+        _lib.check(_lib.lib().vrwkv_groupnorm_gate(y.data_ptr(), gate.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                   y.numel() // C, C, group, float(eps), _DT[y.dtype], _DT[gate.dtype],
+                                                   _stream_ptr(y.device)))
+    return out
