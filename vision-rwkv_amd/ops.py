@@ -293,6 +293,11 @@ POST_NONE, POST_SIGMOID_GATE, POST_RESIDUAL = 0, 1, 2
 ROW_FUSE_ENABLED = True      # set False to make row_fuse run the tensor-op sequence everywhere (for comparisons)
 
 
+def _vec_ok(*tensors):
+    """True when every given tensor can be read as it lies in 16-byte pieces (dense and 16-byte aligned)."""
+    return all(t is None or (t.is_contiguous() and t.data_ptr() % 16 == 0) for t in tensors)
+
+
 def row_fuse_tensor_ops(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NONE, post=POST_NONE, eps=1e-5):
     """The PyTorch-op sequence row_fuse replaces (what the reference runs: vrwkv.py:184-186, :256-261, :300-313);
     used under autograd and wherever the kernel does not apply."""
@@ -321,6 +326,8 @@ def row_fuse(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NO
     a = a.contiguous()
     other = other.contiguous() if other is not None else None
     par = [p.detach().reshape(-1).to(a.dtype).contiguous() if p is not None else None for p in (ln_weight, ln_bias, gamma)]
+    if not _vec_ok(a, other, *par):
+        return row_fuse_tensor_ops(a, other, ln_weight, ln_bias, gamma, pre, post, eps)
     for p in par:
         if p is not None and p.numel() != N:
             raise RuntimeError("LayerNorm weight, bias and gamma must have one element per channel")
@@ -351,6 +358,8 @@ def maa_mix(x, sx, m, maas, maa_table=None):
     if not fits:
         return maa_mix_tensor_ops(x, sx, m, maas)
     x, sx, m = x.contiguous(), sx.contiguous(), m.contiguous()
+    if not _vec_ok(x, sx, m):
+        return maa_mix_tensor_ops(x, sx, m, maas)
     table = maa_table if maa_table is not None else stack_mixes(maas, x.device)
     if tuple(table.shape) != (5, C) or table.dtype != torch.float32 or not table.is_contiguous():
         raise RuntimeError("maa table must be a contiguous float32 (5, C) tensor")
@@ -383,6 +392,8 @@ def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
     y, gate = y.contiguous(), gate.contiguous()
     w = gn_weight.detach().to(gate.dtype).contiguous()
     b = gn_bias.detach().to(gate.dtype).contiguous()
+    if not _vec_ok(y, gate, w, b):
+        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
     out = torch.empty_like(gate)
     with torch.cuda.device(y.device):
         _lib.check(_lib.lib().vrwkv_groupnorm_gate(y.data_ptr(), gate.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(),
