@@ -59,6 +59,30 @@ def test_argument_validation_without_device(lib):
     assert f(one, one, one, one, one, 1, 1 << 20, 1 << 10, 0, None, 0, None) == 3
 
 
+def test_elementwise_entry_points_validate_without_device(lib):
+    """The fused element-wise entry points reject bad arguments before touching the device."""
+    one = ctypes.c_void_p(64)
+    rf = lib.vrwkv_rowfuse
+    assert rf(None, None, None, None, None, one, 4, 64, 0, 0, 1e-5, 1, None) == 1            # a is null
+    assert rf(one, None, None, None, None, one, 4, 64, 0, 1, 1e-5, 1, None) == 1              # gate without `other`
+    assert rf(one, None, one, None, None, one, 4, 64, 0, 0, 1e-5, 1, None) == 1               # LayerNorm weight without bias
+    assert rf(one, None, None, None, None, one, 4, 60, 0, 0, 1e-5, 1, None) == 3              # N not a multiple of 8 (bf16)
+    assert rf(one, None, None, None, None, one, 4, 64, 0, 0, 1e-5, 9, None) == 2              # unknown dtype
+    assert rf(one, None, None, None, None, ctypes.c_void_p(72), 4, 64, 0, 0, 1e-5, 1, None) == 1   # misaligned output
+    assert rf(one, None, None, None, None, one, 4, 64, 2, 0, 1e-5, 1, None) == 1              # unknown pre
+    mm = lib.vrwkv_maa_mix
+    outs = (ctypes.c_void_p * 5)(64, 64, 64, 64, 64)
+    assert mm(one, one, one, one, outs, 0, 64, 1, None) == 1                                    # no rows
+    assert mm(one, one, one, one, outs, 4, 60, 1, None) == 3                                    # C not a multiple of 8
+    outs[3] = None
+    assert mm(one, one, one, one, outs, 4, 64, 1, None) == 1                                    # a null output
+    gg = lib.vrwkv_groupnorm_gate
+    assert gg(one, one, one, one, one, 4, 128, 64, 1e-5, 0, 0, None) == 2                      # fp32 gate / output
+    assert gg(one, one, one, one, one, 4, 128, 48, 1e-5, 0, 1, None) == 3                      # C not a multiple of the group
+    assert gg(one, one, one, one, one, 4, 96, 24, 1e-5, 0, 1, None) == 3                       # group not 8..128 in powers of two
+    assert b"group" in lib.vrwkv_last_error()
+
+
 def test_python_boundary_errors_without_device():
     import torch
     import vision_rwkv_amd as ops
