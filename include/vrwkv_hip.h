@@ -105,6 +105,15 @@ int vrwkv_qshift_mix(const void* x, const float* mix, void* const* out, int n_mi
                      int B, int T, int C, int Hp, int Wp, int shift_pixel, int quarter_width,
                      int head_dim, int io_dtype, void* hip_stream);
 
+/* Backward of vrwkv_qshift_mix (the reference differentiates its PyTorch ops by autograd; no native code):
+ * gout[m]: gradients of out[m], (B,T,C) of io_dtype; gx: (B,T,C) of io_dtype; gmix: (n_mix, C) fp32, summed over
+ * batch and tokens in a fixed order.  workspace: vrwkv_qshift_mix_bwd_workspace_bytes(n_mix, B, T, C) bytes. */
+size_t vrwkv_qshift_mix_bwd_workspace_bytes(int n_mix, int B, int T, int C);
+int vrwkv_qshift_mix_bwd(const void* x, const float* mix, const void* const* gout, int n_mix,
+                         void* gx, float* gmix, int B, int T, int C, int Hp, int Wp, int shift_pixel,
+                         int quarter_width, int head_dim, int io_dtype,
+                         void* workspace, size_t workspace_bytes, void* hip_stream);
+
 /* ---- fused row-wise epilogues of the blocks (the elementwise steps behind the operator and the GEMMs) ----
  * For every row of N channels:  y = LayerNorm(pre(a)) (weight, bias; LayerNorm skipped when ln_weight is NULL),
  * out = y (post 0) | sigmoid(other) * y (post 1) | other + gamma * y (post 2, gamma NULL = 1); pre 0 = identity,

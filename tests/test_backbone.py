@@ -274,3 +274,37 @@ def test_vrwkv6_mix_kernels_against_tensor_ops(B, T, C, dtype):
     xg = x.float().requires_grad_(True)
     sum(o.sum() for o in ops.maa_mix(xg, sx.float(), m.float(), [a.float() for a in maas])).backward()
     assert xg.grad is not None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,Hp,Wp,C,head_dim,cls,dtype", [(2, 3, 5, 16, 0, False, torch.float32), (2, 14, 14, 192, 0, False, torch.float32),
+                                                           (1, 7, 9, 22, 0, False, torch.float32), (2, 6, 4, 128, 64, True, torch.float32),
+                                                           (2, 14, 14, 768, 0, False, torch.bfloat16), (3, 5, 3, 8, 0, False, torch.float32)])
+def test_fused_qshift_mix_backward_against_autograd(B, Hp, Wp, C, head_dim, cls, dtype):
+    """Gradients of the fused q_shift + mix (hand-written backward kernel) against autograd through the tensor-op
+    formulation evaluated in float64 on the same inputs: grad of x and of every mix vector, three / two / one mix,
+    per-head quarters with a trailing class token, a channel count that forces the scalar path.
+    Tolerance: 1e-5 of the gradient's scale for fp32 I/O, 2e-2 for bf16 (one rounding of gx, bf16 inputs)."""
+    import vision_rwkv_amd as ops
+    from vision_rwkv_amd.backbone6 import q_shift_multihead
+    dev = "cuda:0"
+    torch.manual_seed(Hp * Wp + C)
+    T = Hp * Wp + (1 if cls else 0)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for n_mix in (3, 2, 1):
+        x = torch.randn(B, T, C, device=dev).to(dtype).requires_grad_(True)
+        mixes = [torch.rand(1, 1, C, device=dev).requires_grad_(True) for _ in range(n_mix)]
+        gouts = [torch.randn(B, T, C, device=dev).to(dtype) for _ in range(n_mix)]
+        outs = ops.q_shift_mix_autograd(x, mixes, 1, 0.25, (Hp, Wp), head_dim)
+        torch.autograd.backward(outs, gouts)
+        xr = x.detach().double().requires_grad_(True)
+        mr = [m.detach().double().requires_grad_(True) for m in mixes]
+        sx = (q_shift_multihead(xr, 1, head_dim, (Hp, Wp), cls) if head_dim else ops.q_shift(xr, 1, 0.25, (Hp, Wp)))
+        ref = [xr * m + sx * (1 - m) for m in mr]
+        torch.autograd.backward(ref, [g.double() for g in gouts])
+        for o, r in zip(outs, ref):
+            assert (o.double() - r).abs().max().item() <= tol * r.abs().max().item()
+        assert (x.grad.double() - xr.grad).abs().max().item() <= tol * xr.grad.abs().max().item()
+        for m, r in zip(mixes, mr):
+            assert m.grad.shape == m.shape
+            assert (m.grad.double() - r.grad).abs().max().item() <= tol * max(r.grad.abs().max().item(), 1.0)

@@ -61,6 +61,10 @@ def _declare(lib):
     lib.vrwkv_wkv6_bwd.restype = i
     lib.vrwkv_qshift_mix.argtypes = [vp, fp, c.POINTER(c.c_void_p), i, i, i, i, i, i, i, i, i, i, vp]
     lib.vrwkv_qshift_mix.restype = i
+    lib.vrwkv_qshift_mix_bwd_workspace_bytes.argtypes = [i, i, i, i]
+    lib.vrwkv_qshift_mix_bwd_workspace_bytes.restype = sz
+    lib.vrwkv_qshift_mix_bwd.argtypes = [vp, fp, c.POINTER(c.c_void_p), i, vp, fp, i, i, i, i, i, i, i, i, i, vp, sz, vp]
+    lib.vrwkv_qshift_mix_bwd.restype = i
     lib.vrwkv_rowfuse.argtypes = [vp, vp, vp, vp, vp, vp, c.c_longlong, i, i, i, c.c_float, i, vp]
     lib.vrwkv_rowfuse.restype = i
     lib.vrwkv_maa_mix.argtypes = [vp, vp, vp, fp, c.POINTER(c.c_void_p), c.c_longlong, i, i, vp]

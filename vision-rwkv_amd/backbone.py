@@ -14,7 +14,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .ops import (RUN_CUDA, bi_wkv_forward, q_shift, q_shift_mix, stack_mixes, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE, POST_SIGMOID_GATE,
+from .ops import (RUN_CUDA, bi_wkv_forward, q_shift, q_shift_mix, q_shift_mix_autograd, stack_mixes, row_fuse, PRE_NONE, PRE_RELU_SQ, POST_NONE, POST_SIGMOID_GATE,
                   POST_RESIDUAL)
 
 
@@ -47,8 +47,11 @@ def eval_cached(module, name, params, extra, make):
 
 
 def _mix(module, x, mixes, shift_pixel, gamma, patch_resolution, fused, head_dim=0):
-    """[x*m + q_shift(x)*(1-m) for m in mixes]: one fused kernel at inference, tensor ops under autograd."""
-    if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or mixes[0].requires_grad)):
+    """[x*m + q_shift(x)*(1-m) for m in mixes]: one fused kernel (forward, and backward under autograd); tensor ops
+    when `fused` is off or the tensors are not on the GPU."""
+    if fused and x.is_cuda:
+        if torch.is_grad_enabled() and (x.requires_grad or any(m.requires_grad for m in mixes)):
+            return q_shift_mix_autograd(x, mixes, shift_pixel, gamma, patch_resolution, head_dim)
         table = eval_cached(module, "mix_table", mixes, x.device, lambda: stack_mixes(mixes, x.device))
         return q_shift_mix(x.contiguous(), mixes, shift_pixel, gamma, patch_resolution, head_dim, mix_table=table)
     xx = q_shift(x, shift_pixel, gamma, patch_resolution)

@@ -11,7 +11,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .backbone import VRWKV, eval_cached
-from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, stack_mixes, row_fuse, maa_mix, groupnorm_gate, PRE_NONE, PRE_RELU_SQ, POST_NONE,
+from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, q_shift_mix_autograd, stack_mixes, row_fuse, maa_mix, groupnorm_gate, PRE_NONE, PRE_RELU_SQ, POST_NONE,
                   POST_SIGMOID_GATE, POST_RESIDUAL)
 
 
@@ -28,9 +28,12 @@ def q_shift_multihead(x, shift_pixel=1, head_dim=HEAD_SIZE, patch_resolution=Non
 
 
 def _shift_and_mix(module, x, mixes, shift_pixel, patch_resolution, with_cls_token, fused, params):
-    """[x*m + shift(x)*(1-m) for m in mixes()]; one HIP kernel at inference, tensor ops under autograd.  `mixes` is a
-    callable (the vectors may be derived from `params`); at inference its stacked fp32 table is kept on the module."""
-    if fused and x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or params[0].requires_grad)):
+    """[x*m + shift(x)*(1-m) for m in mixes()]; one HIP kernel (forward, and backward under autograd), tensor ops when
+    `fused` is off or off the GPU.  `mixes` is a callable (the vectors may be derived from `params`); at inference
+    its stacked fp32 table is kept on the module."""
+    if fused and x.is_cuda:
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in params)):
+            return q_shift_mix_autograd(x, mixes(), shift_pixel, 1 / 4, patch_resolution, HEAD_SIZE)
         table = eval_cached(module, "mix_table", params, x.device, lambda: stack_mixes(mixes(), x.device))
         return q_shift_mix(x.contiguous(), [None] * table.shape[0], shift_pixel, 1 / 4, patch_resolution,
                            head_dim=HEAD_SIZE, mix_table=table)

@@ -8,6 +8,13 @@
 // takes its value from the pixel one step left / right / up / down (zero outside the grid);
 // channels >= 4g pass through.  q_shift_multihead (vrwkv6.py:75-100) is the same with the quarter
 // taken inside every head: pass head_dim = 64 (0 = whole-tensor quarters).
+//
+// Backward (the reference differentiates the PyTorch ops by autograd): with g_m the gradient of out_m,
+//   gx[b,t,c]  = sum_m g_m[b,t,c] mix_m[c]  +  sum_m g_m[b,t',c] (1 - mix_m[c])     t' = the token that reads t
+//   gmix_m[c]  = sum_{b,t} g_m[b,t,c] (x[b,t,c] - xx[b,t,c])
+// (t' is one step right / left / down / up of t, none at the border; pass-through channels and a trailing class
+// token read themselves).  One kernel writes gx and per-(batch, token-chunk) partial sums of gmix, which
+// batch_sum_kernel then adds in a fixed order.
 #include "vrwkv_common.h"
 
 namespace vrwkv {
@@ -56,6 +63,122 @@ void qshift_mix_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_
         }
         store_vec<IO, VEC>(outs[m] + row + c, r);
     }
+}
+
+constexpr int QS_TCH = 14;       // tokens a thread walks in the backward kernel (one partial gmix row per chunk)
+
+// direction of a channel vector and the token offsets of its source (forward) / destination (backward)
+__device__ __forceinline__ int qs_dir(int c, int g, int head_dim) {
+    const int cq = head_dim > 0 ? c % head_dim : c;
+    return (g > 0 && cq < 4 * g) ? cq / g : 4;
+}
+// token that the forward reads for (t, dir): -1 = zero fill, t itself for pass-through
+__device__ __forceinline__ int qs_src(int t, int dir, int Hp, int Wp, int shift, int n_grid) {
+    if (t >= n_grid || dir == 4) return t;
+    const int yy = t / Wp, xc = t % Wp;
+    int sy = yy, sx = xc;
+    if (dir == 0) sx = xc - shift; else if (dir == 1) sx = xc + shift;
+    else if (dir == 2) sy = yy - shift; else sy = yy + shift;
+    return (sx >= 0 && sx < Wp && sy >= 0 && sy < Hp) ? sy * Wp + sx : -1;
+}
+// token whose forward value was read from (t, dir): the opposite step
+__device__ __forceinline__ int qs_dst(int t, int dir, int Hp, int Wp, int shift, int n_grid) {
+    if (t >= n_grid || dir == 4) return t;
+    const int yy = t / Wp, xc = t % Wp;
+    int sy = yy, sx = xc;
+    if (dir == 0) sx = xc + shift; else if (dir == 1) sx = xc - shift;
+    else if (dir == 2) sy = yy + shift; else sy = yy - shift;
+    return (sx >= 0 && sx < Wp && sy >= 0 && sy < Hp) ? sy * Wp + sx : -1;
+}
+
+template <typename IO, int VEC, int NMIX>
+__global__ __launch_bounds__(256)
+void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_, const IO* __restrict__ g0,
+                           const IO* __restrict__ g1, const IO* __restrict__ g2, IO* __restrict__ gx_,
+                           float* __restrict__ gmix_part, int T, int C, int Hp, int Wp, int shift, int g, int head_dim,
+                           int n_grid_tokens, int n_tchunk)
+{
+    const int cv = blockIdx.x * blockDim.x + threadIdx.x;
+    const int c = cv * VEC;
+    if (c >= C) return;
+    const int tc = blockIdx.y, b = blockIdx.z;
+    const int dir = qs_dir(c, g, head_dim);
+    const IO* gs[3] = {g0, g1, g2};
+    float mu[NMIX][VEC], acc[NMIX][VEC];
+#pragma unroll
+    for (int m = 0; m < NMIX; ++m)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { mu[m][e] = mix_[(size_t)m * C + c + e]; acc[m][e] = 0.f; }
+    const size_t slab = (size_t)b * T * C + c;
+    const int t_end = min(T, (tc + 1) * QS_TCH);
+    for (int t = tc * QS_TCH; t < t_end; ++t) {
+        const int ts = qs_src(t, dir, Hp, Wp, shift, n_grid_tokens);
+        const int td = qs_dst(t, dir, Hp, Wp, shift, n_grid_tokens);
+        float xs[VEC], xx[VEC], gx[VEC];
+        load_vec<IO, VEC>(x_ + slab + (size_t)t * C, xs);
+        if (ts >= 0 && ts != t) load_vec<IO, VEC>(x_ + slab + (size_t)ts * C, xx);
+        else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xx[e] = ts >= 0 ? xs[e] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
+#pragma unroll
+        for (int m = 0; m < NMIX; ++m) {
+            float gt[VEC], gd[VEC];
+            load_vec<IO, VEC>(gs[m] + slab + (size_t)t * C, gt);
+            if (td >= 0 && td != t) load_vec<IO, VEC>(gs[m] + slab + (size_t)td * C, gd);
+            else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gd[e] = td >= 0 ? gt[e] : 0.f;
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                gx[e] = fmaf(gt[e], mu[m][e], fmaf(gd[e], 1.f - mu[m][e], gx[e]));
+                acc[m][e] = fmaf(gt[e], xs[e] - xx[e], acc[m][e]);
+            }
+        }
+        store_vec<IO, VEC>(gx_ + slab + (size_t)t * C, gx);
+    }
+    float* part = gmix_part + ((size_t)b * n_tchunk + tc) * NMIX * C + c;
+#pragma unroll
+    for (int m = 0; m < NMIX; ++m)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) part[(size_t)m * C + e] = acc[m][e];
+}
+
+template <typename IO, int VEC>
+int launch_bwd(const void* x, const float* mix, const void* const* gout, void* gx, float* gmix, float* part, int n_mix,
+               int B, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid, hipStream_t st) {
+    const int ncv = C / VEC;
+    const int n_tchunk = (T + QS_TCH - 1) / QS_TCH;
+    const dim3 block(ncv < 256 ? ((ncv + 63) / 64) * 64 : 256);
+    const dim3 grid((ncv + block.x - 1) / block.x, n_tchunk, B);
+    const IO* xx = static_cast<const IO*>(x);
+    const IO* g0 = static_cast<const IO*>(gout[0]);
+    const IO* g1 = n_mix > 1 ? static_cast<const IO*>(gout[1]) : nullptr;
+    const IO* g2 = n_mix > 2 ? static_cast<const IO*>(gout[2]) : nullptr;
+    IO* pgx = static_cast<IO*>(gx);
+    switch (n_mix) {
+        case 1: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
+        case 2: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
+        case 3: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
+    }
+    // gmix[m][c] = sum over the B * n_tchunk partial rows: the rows are (n_mix * C) wide
+    const int wide = n_mix * C;
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gmix, (const float*)nullptr,
+                       (float*)nullptr, B * n_tchunk, wide);
+    return check_launch("qshift_mix_bwd");
+}
+
+template <typename IO>
+int launch_bwd_io(const void* x, const float* mix, const void* const* gout, void* gx, float* gmix, float* part, int n_mix,
+                  int B, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid, bool vec_ok, hipStream_t st) {
+    constexpr int V = 16 / sizeof(IO);
+    const int period = head_dim > 0 ? head_dim : C;
+    if (vec_ok && C % V == 0 && g % V == 0 && period % V == 0)
+        return launch_bwd<IO, V>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift, g, head_dim, n_grid, st);
+    return launch_bwd<IO, 1>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift, g, head_dim, n_grid, st);
 }
 
 template <typename IO, int VEC>
@@ -131,6 +254,62 @@ extern "C" int vrwkv_qshift_mix(const void* x, const float* mix, void* const* ou
         case VRWKV_F32:  return launch_io<float>(x, mix, out, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
         case VRWKV_BF16: return launch_io<__hip_bfloat16>(x, mix, out, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
         case VRWKV_F16:  return launch_io<__half>(x, mix, out, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
+    }
+    return VRWKV_UNSUPPORTED_DTYPE;
+}
+
+extern "C" size_t vrwkv_qshift_mix_bwd_workspace_bytes(int n_mix, int B, int T, int C) {
+    if (n_mix < 1 || n_mix > 3 || B <= 0 || T <= 0 || C <= 0) return 0;
+    return (size_t)B * ((T + QS_TCH - 1) / QS_TCH) * n_mix * C * sizeof(float);
+}
+
+extern "C" int vrwkv_qshift_mix_bwd(const void* x, const float* mix, const void* const* gout, int n_mix,
+                                    void* gx, float* gmix, int B, int T, int C, int Hp, int Wp, int shift_pixel,
+                                    int quarter_width, int head_dim, int io_dtype,
+                                    void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (B <= 0 || T <= 0 || C <= 0 || Hp <= 0 || Wp <= 0 || n_mix < 1 || n_mix > 3 || shift_pixel < 0) {
+        set_error("qshift_mix_bwd: bad sizes (B=%d T=%d C=%d Hp=%d Wp=%d n_mix=%d shift=%d)", B, T, C, Hp, Wp, n_mix, shift_pixel);
+        return VRWKV_INVALID_ARG;
+    }
+    const int n_grid = Hp * Wp;
+    if (n_grid != T && n_grid != T - 1) {
+        set_error("qshift_mix_bwd: Hp*Wp must be T or T-1 (got %d*%d, T=%d)", Hp, Wp, T);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    if (quarter_width < 0 || head_dim < 0 || (head_dim > 0 && (C % head_dim || 4 * quarter_width > head_dim)) ||
+        (head_dim == 0 && 4 * (long long)quarter_width > C)) {
+        set_error("qshift_mix_bwd: quarter_width=%d does not fit (C=%d, head_dim=%d)", quarter_width, C, head_dim);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    if (T > 65535 * QS_TCH || B > 65535) {
+        set_error("qshift_mix_bwd: B must be <= 65535 and T <= %d", 65535 * QS_TCH);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    if (io_dtype != VRWKV_F32 && io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16) {
+        set_error("qshift_mix_bwd: unsupported io_dtype code %d", io_dtype);
+        return VRWKV_UNSUPPORTED_DTYPE;
+    }
+    if (!x || !mix || !gout || !gx || !gmix) {
+        set_error("qshift_mix_bwd: null pointer argument");
+        return VRWKV_INVALID_ARG;
+    }
+    uintptr_t bits = (uintptr_t)x | (uintptr_t)gx;
+    for (int m = 0; m < n_mix; ++m) {
+        if (!gout[m]) { set_error("qshift_mix_bwd: null gradient pointer %d", m); return VRWKV_INVALID_ARG; }
+        bits |= (uintptr_t)gout[m];
+    }
+    const size_t need = vrwkv_qshift_mix_bwd_workspace_bytes(n_mix, B, T, C);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 3)) {
+        set_error("qshift_mix_bwd: a 4-byte aligned workspace of %zu bytes is required", need);
+        return VRWKV_WORKSPACE_TOO_SMALL;
+    }
+    const bool vec_ok = (bits & 15) == 0;
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    float* part = static_cast<float*>(workspace);
+    switch (io_dtype) {
+        case VRWKV_F32:  return launch_bwd_io<float>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
+        case VRWKV_BF16: return launch_bwd_io<__hip_bfloat16>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
+        case VRWKV_F16:  return launch_bwd_io<__half>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift_pixel, quarter_width, head_dim, n_grid, vec_ok, st);
     }
     return VRWKV_UNSUPPORTED_DTYPE;
 }

@@ -400,3 +400,49 @@ def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
                                                    y.numel() // C, C, group, float(eps), _DT[y.dtype], _DT[gate.dtype],
                                                    _stream_ptr(y.device)))
     return out
+
+
+class _QShiftMix(torch.autograd.Function):
+    """q_shift + mix lerps with a hand-written backward (vrwkv_qshift_mix / vrwkv_qshift_mix_bwd); the mix vectors
+    enter as one (n_mix, C) fp32 table, so whatever produced them (parameters, 1 - parameter, ...) is differentiated
+    by autograd outside."""
+
+    @staticmethod
+    def forward(ctx, x, table, shift_pixel, gamma, Hp, Wp, head_dim):
+        x = x.contiguous()
+        table = table.contiguous()
+        ctx.save_for_backward(x, table)
+        ctx.meta = (shift_pixel, gamma, Hp, Wp, head_dim)
+        outs = q_shift_mix(x, [None] * table.shape[0], shift_pixel, gamma, (Hp, Wp), head_dim, mix_table=table)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        x, table = ctx.saved_tensors
+        shift_pixel, gamma, Hp, Wp, head_dim = ctx.meta
+        B, T, C = x.shape
+        n_mix = table.shape[0]
+        gs = [g.to(x.dtype).contiguous() for g in gouts]
+        gx = torch.empty_like(x)
+        gmix = torch.empty_like(table)
+        L = _lib.lib()
+        ws_bytes = L.vrwkv_qshift_mix_bwd_workspace_bytes(n_mix, B, T, C)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        ptrs = (ctypes.c_void_p * n_mix)(*[g.data_ptr() for g in gs])
+        g = head_dim // 4 if head_dim else int(C * gamma)
+        with torch.cuda.device(x.device):
+            _lib.check(L.vrwkv_qshift_mix_bwd(x.data_ptr(), table.data_ptr(), ptrs, n_mix, gx.data_ptr(), gmix.data_ptr(),
+                                              B, T, C, Hp, Wp, shift_pixel, g, head_dim, _DT[x.dtype],
+                                              ws.data_ptr(), ws_bytes, _stream_ptr(x.device)))
+        return gx, gmix, None, None, None, None, None
+
+
+def q_shift_mix_autograd(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, head_dim=0):
+    """q_shift_mix for training: the same fused forward kernel, and one fused backward kernel in place of autograd
+    through the slice copies and lerps.  `mixes` may be parameters or tensors derived from parameters."""
+    _check_input(x, "x")
+    if x.dim() != 3 or x.dtype not in _DT:
+        raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
+    table = torch.stack([m.reshape(-1).float() for m in mixes])
+    Hp, Wp = patch_resolution
+    return list(_QShiftMix.apply(x, table, shift_pixel, gamma, Hp, Wp, head_dim))
