@@ -65,7 +65,8 @@ void qshift_mix_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_
     }
 }
 
-constexpr int QS_TCH = 14;       // tokens a thread walks in the backward kernel (one partial gmix row per chunk)
+constexpr int QS_CX = 32, QS_TY = 8;   // backward workgroup: 32 channel vectors x 8 token lanes
+constexpr int QS_TCH = 32;             // tokens per workgroup (one partial gmix row per chunk): 4 per thread
 
 // direction of a channel vector and the token offsets of its source (forward) / destination (backward)
 __device__ __forceinline__ int qs_dir(int c, int g, int head_dim) {
@@ -92,59 +93,72 @@ __device__ __forceinline__ int qs_dst(int t, int dir, int Hp, int Wp, int shift,
 }
 
 template <typename IO, int VEC, int NMIX>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(QS_CX * QS_TY)
 void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_, const IO* __restrict__ g0,
                            const IO* __restrict__ g1, const IO* __restrict__ g2, IO* __restrict__ gx_,
                            float* __restrict__ gmix_part, int T, int C, int Hp, int Wp, int shift, int g, int head_dim,
                            int n_grid_tokens, int n_tchunk)
 {
-    const int cv = blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ float s_acc[QS_TY][NMIX][QS_CX * VEC];
+    const int cx = threadIdx.x % QS_CX, ty = threadIdx.x / QS_CX;
+    const int cv = blockIdx.x * QS_CX + cx;
     const int c = cv * VEC;
-    if (c >= C) return;
+    const bool cok = c < C;
     const int tc = blockIdx.y, b = blockIdx.z;
-    const int dir = qs_dir(c, g, head_dim);
+    const int dir = qs_dir(cok ? c : 0, g, head_dim);
     const IO* gs[3] = {g0, g1, g2};
     float mu[NMIX][VEC], acc[NMIX][VEC];
 #pragma unroll
     for (int m = 0; m < NMIX; ++m)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) { mu[m][e] = mix_[(size_t)m * C + c + e]; acc[m][e] = 0.f; }
+        for (int e = 0; e < VEC; ++e) { mu[m][e] = cok ? mix_[(size_t)m * C + c + e] : 0.f; acc[m][e] = 0.f; }
     const size_t slab = (size_t)b * T * C + c;
-    const int t_end = min(T, (tc + 1) * QS_TCH);
-    for (int t = tc * QS_TCH; t < t_end; ++t) {
-        const int ts = qs_src(t, dir, Hp, Wp, shift, n_grid_tokens);
-        const int td = qs_dst(t, dir, Hp, Wp, shift, n_grid_tokens);
-        float xs[VEC], xx[VEC], gx[VEC];
-        load_vec<IO, VEC>(x_ + slab + (size_t)t * C, xs);
-        if (ts >= 0 && ts != t) load_vec<IO, VEC>(x_ + slab + (size_t)ts * C, xx);
-        else {
+    if (cok) {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) xx[e] = ts >= 0 ? xs[e] : 0.f;
-        }
+        for (int i = 0; i < QS_TCH / QS_TY; ++i) {
+            const int t = tc * QS_TCH + ty + QS_TY * i;
+            if (t >= T) continue;
+            const int ts = qs_src(t, dir, Hp, Wp, shift, n_grid_tokens);
+            const int td = qs_dst(t, dir, Hp, Wp, shift, n_grid_tokens);
+            // neighbours outside the grid are read from the token itself and masked: no divergent branches, so all
+            // loads of a token are in flight together
+            float xs[VEC], xx[VEC], gx[VEC], gt[NMIX][VEC], gd[NMIX][VEC];
+            load_vec<IO, VEC>(x_ + slab + (size_t)t * C, xs);
+            load_vec<IO, VEC>(x_ + slab + (size_t)(ts >= 0 ? ts : t) * C, xx);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
-#pragma unroll
-        for (int m = 0; m < NMIX; ++m) {
-            float gt[VEC], gd[VEC];
-            load_vec<IO, VEC>(gs[m] + slab + (size_t)t * C, gt);
-            if (td >= 0 && td != t) load_vec<IO, VEC>(gs[m] + slab + (size_t)td * C, gd);
-            else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) gd[e] = td >= 0 ? gt[e] : 0.f;
+            for (int m = 0; m < NMIX; ++m) {
+                load_vec<IO, VEC>(gs[m] + slab + (size_t)t * C, gt[m]);
+                load_vec<IO, VEC>(gs[m] + slab + (size_t)(td >= 0 ? td : t) * C, gd[m]);
             }
+            const float keep_s = ts >= 0 ? 1.f : 0.f, keep_d = td >= 0 ? 1.f : 0.f;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                gx[e] = fmaf(gt[e], mu[m][e], fmaf(gd[e], 1.f - mu[m][e], gx[e]));
-                acc[m][e] = fmaf(gt[e], xs[e] - xx[e], acc[m][e]);
-            }
+            for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
+#pragma unroll
+            for (int m = 0; m < NMIX; ++m)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    gx[e] = fmaf(gt[m][e], mu[m][e], fmaf(keep_d * gd[m][e], 1.f - mu[m][e], gx[e]));
+                    acc[m][e] = fmaf(gt[m][e], xs[e] - keep_s * xx[e], acc[m][e]);
+                }
+            store_vec<IO, VEC>(gx_ + slab + (size_t)t * C, gx);
         }
-        store_vec<IO, VEC>(gx_ + slab + (size_t)t * C, gx);
     }
-    float* part = gmix_part + ((size_t)b * n_tchunk + tc) * NMIX * C + c;
+    // the eight token lanes' sums of a column are added in a fixed order and written as one partial row
 #pragma unroll
     for (int m = 0; m < NMIX; ++m)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) part[(size_t)m * C + e] = acc[m][e];
+        for (int e = 0; e < VEC; ++e) s_acc[ty][m][cx * VEC + e] = acc[m][e];
+    __syncthreads();
+    float* part = gmix_part + ((size_t)b * n_tchunk + tc) * NMIX * C;
+    for (int o = threadIdx.x; o < NMIX * QS_CX * VEC; o += QS_CX * QS_TY) {
+        const int m = o / (QS_CX * VEC), col = o % (QS_CX * VEC);
+        const int cg = blockIdx.x * QS_CX * VEC + col;
+        if (cg >= C) continue;
+        float sum = 0.f;
+#pragma unroll
+        for (int y = 0; y < QS_TY; ++y) sum += s_acc[y][m][col];
+        part[(size_t)m * C + cg] = sum;
+    }
 }
 
 template <typename IO, int VEC>
@@ -152,8 +166,8 @@ int launch_bwd(const void* x, const float* mix, const void* const* gout, void* g
                int B, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid, hipStream_t st) {
     const int ncv = C / VEC;
     const int n_tchunk = (T + QS_TCH - 1) / QS_TCH;
-    const dim3 block(ncv < 256 ? ((ncv + 63) / 64) * 64 : 256);
-    const dim3 grid((ncv + block.x - 1) / block.x, n_tchunk, B);
+    const dim3 block(QS_CX * QS_TY);
+    const dim3 grid((ncv + QS_CX - 1) / QS_CX, n_tchunk, B);
     const IO* xx = static_cast<const IO*>(x);
     const IO* g0 = static_cast<const IO*>(gout[0]);
     const IO* g1 = n_mix > 1 ? static_cast<const IO*>(gout[1]) : nullptr;
