@@ -76,6 +76,16 @@ def test_elementwise_entry_points_validate_without_device(lib):
     assert mm(one, one, one, one, outs, 4, 60, 1, None) == 3                                    # C not a multiple of 8
     outs[3] = None
     assert mm(one, one, one, one, outs, 4, 64, 1, None) == 1                                    # a null output
+    qb = lib.vrwkv_qshift_mix_bwd
+    gp = (ctypes.c_void_p * 3)(64, 64, 64)
+    need = lib.vrwkv_qshift_mix_bwd_workspace_bytes(3, 2, 196, 768)
+    assert need == 2 * 7 * 3 * 768 * 4                                                        # one partial row per 32 tokens
+    assert qb(one, one, gp, 3, one, one, 2, 196, 768, 14, 14, 1, 192, 0, 1, None, 0, None) == 5     # workspace missing
+    assert b"workspace" in lib.vrwkv_last_error()
+    assert qb(one, one, gp, 3, one, one, 2, 196, 768, 13, 14, 1, 192, 0, 1, one, need, None) == 3   # grid does not match T
+    assert qb(one, one, gp, 4, one, one, 2, 196, 768, 14, 14, 1, 192, 0, 1, one, need, None) == 1   # n_mix out of range
+    gp[1] = None
+    assert qb(one, one, gp, 3, one, one, 2, 196, 768, 14, 14, 1, 192, 0, 1, one, need, None) == 1   # a null gradient
     gg = lib.vrwkv_groupnorm_gate
     assert gg(one, one, one, one, one, 4, 128, 64, 1e-5, 0, 0, None) == 2                      # fp32 gate / output
     assert gg(one, one, one, one, one, 4, 128, 48, 1e-5, 0, 1, None) == 3                      # C not a multiple of the group
