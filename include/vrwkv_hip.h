@@ -126,6 +126,18 @@ int vrwkv_rowfuse(const void* a, const void* other, const void* ln_weight, const
                   const void* gamma, void* out, long long rows, int N, int pre, int post, float eps,
                   int io_dtype, void* hip_stream);
 
+/* Backward of vrwkv_rowfuse (the reference differentiates its PyTorch ops by autograd; no native code).
+ * gout: gradient of out; ga: gradient of a; gother: gradient of `other` for the sigmoid gate (for the residual it is
+ * gout itself and nothing is written; may be NULL then); gparam: (3, N) fp32 = gradients of ln_weight, ln_bias and
+ * gamma summed over the rows in a fixed order (required when LayerNorm or gamma take part; rows unused by the call
+ * are zero).  With LayerNorm or gamma N is at most 1024.  workspace: vrwkv_rowfuse_bwd_workspace_bytes(rows, N)
+ * bytes, needed only when gparam is. */
+size_t vrwkv_rowfuse_bwd_workspace_bytes(long long rows, int N);
+int vrwkv_rowfuse_bwd(const void* a, const void* other, const void* ln_weight, const void* ln_bias,
+                      const void* gamma, const void* gout, void* ga, void* gother, float* gparam,
+                      long long rows, int N, int pre, int post, float eps, int io_dtype,
+                      void* workspace, size_t workspace_bytes, void* hip_stream);
+
 /* ---- element-wise steps of the VRWKV6 spatial mix (.../backbones/vrwkv6.py:176-212), one pass each ----
  * vrwkv_maa_mix: the five data-dependent token mixes of jit_func (:190-194),
  *   out[i] = x + (sx - x) * (maa[i] + m[i]),  i = w, k, v, r, g;

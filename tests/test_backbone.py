@@ -308,3 +308,48 @@ def test_fused_qshift_mix_backward_against_autograd(B, Hp, Wp, C, head_dim, cls,
         for m, r in zip(mixes, mr):
             assert m.grad.shape == m.shape
             assert (m.grad.double() - r.grad).abs().max().item() <= tol * max(r.grad.abs().max().item(), 1.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,dtype,with_sums", [(768, torch.float32, True), (1024, torch.float32, True), (64, torch.float32, True),
+                                                (768, torch.bfloat16, True), (4096, torch.float32, False),
+                                                (3072, torch.bfloat16, False)])
+def test_row_fuse_backward_against_autograd(N, dtype, with_sums):
+    """Gradients of the fused row epilogues (hand-written backward kernel) against autograd through the tensor-op
+    sequence in float64 on the same inputs: every pre / LayerNorm / post combination, 45 rows (the last workgroup and
+    the last wave's run of rows are partial).  Rows longer than 1024 channels are differentiated by the kernel only
+    without LayerNorm and gamma.  Tolerance: 2e-4 of each gradient's scale for fp32 I/O (fast exp / rcp in the gate,
+    fp32 sums over rows), 3e-2 for bf16."""
+    import vision_rwkv_amd as ops
+    O = ops.ops
+    dev = "cuda:0"
+    torch.manual_seed(N)
+    rows = (5, 9)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    combos = [(O.PRE_NONE, O.POST_SIGMOID_GATE, False, False), (O.PRE_RELU_SQ, O.POST_NONE, False, False),
+              (O.PRE_NONE, O.POST_RESIDUAL, False, False)]
+    if with_sums:
+        combos += [(O.PRE_NONE, O.POST_SIGMOID_GATE, True, False), (O.PRE_RELU_SQ, O.POST_NONE, True, False),
+                   (O.PRE_NONE, O.POST_RESIDUAL, True, True), (O.PRE_NONE, O.POST_RESIDUAL, False, True),
+                   (O.PRE_NONE, O.POST_NONE, True, False), (O.PRE_RELU_SQ, O.POST_SIGMOID_GATE, True, False)]
+    for pre, post, ln, use_gamma in combos:
+        a = torch.randn(*rows, N, device=dev).to(dtype).requires_grad_(True)
+        o = torch.randn(*rows, N, device=dev).to(dtype).requires_grad_(True) if post else None
+        w = (1 + 0.3 * torch.randn(N, device=dev)).to(dtype).requires_grad_(True) if ln else None
+        b = (0.3 * torch.randn(N, device=dev)).to(dtype).requires_grad_(True) if ln else None
+        gm = torch.randn(N, device=dev).to(dtype).requires_grad_(True) if use_gamma else None
+        gout = torch.randn(*rows, N, device=dev).to(dtype)
+        out = ops.row_fuse(a, o, w, b, gm, pre, post)
+        assert out.grad_fn is not None and "RowFuse" in type(out.grad_fn).__name__
+        out.backward(gout)
+        d = lambda t: t.detach().double().requires_grad_(True) if t is not None else None
+        a2, o2, w2, b2, g2 = d(a), d(o), d(w), d(b), d(gm)
+        ref = O.row_fuse_tensor_ops(a2, o2, w2, b2, g2, pre, post)
+        ref.backward(gout.double())
+        assert (out.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+        for name, t, r in (("a", a, a2), ("other", o, o2), ("weight", w, w2), ("bias", b, b2), ("gamma", gm, g2)):
+            if t is None:
+                continue
+            assert t.grad is not None, (name, pre, post, ln)
+            err = (t.grad.double() - r.grad).abs().max().item() / max(r.grad.abs().max().item(), 1e-6)
+            assert err <= tol, (name, pre, post, ln, use_gamma, err)

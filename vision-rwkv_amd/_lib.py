@@ -67,6 +67,10 @@ def _declare(lib):
     lib.vrwkv_qshift_mix_bwd.restype = i
     lib.vrwkv_rowfuse.argtypes = [vp, vp, vp, vp, vp, vp, c.c_longlong, i, i, i, c.c_float, i, vp]
     lib.vrwkv_rowfuse.restype = i
+    lib.vrwkv_rowfuse_bwd_workspace_bytes.argtypes = [c.c_longlong, i]
+    lib.vrwkv_rowfuse_bwd_workspace_bytes.restype = sz
+    lib.vrwkv_rowfuse_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, fp, c.c_longlong, i, i, i, c.c_float, i, vp, sz, vp]
+    lib.vrwkv_rowfuse_bwd.restype = i
     lib.vrwkv_maa_mix.argtypes = [vp, vp, vp, fp, c.POINTER(c.c_void_p), c.c_longlong, i, i, vp]
     lib.vrwkv_maa_mix.restype = i
     lib.vrwkv_groupnorm_gate.argtypes = [vp, vp, vp, vp, vp, c.c_longlong, i, i, c.c_float, i, i, vp]

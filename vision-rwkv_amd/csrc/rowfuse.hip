@@ -9,6 +9,16 @@
 //   :300-313  x = x + gamma * ln(att(x)) / x + gamma * att(ln(x))  -> a = branch output, other = x, (LayerNorm,) gamma
 // One wave per row: a lane keeps its 16-byte vectors of the row in registers (read once), the mean and the variance are
 // reduced across the wave in fp32 (two passes over the registers), the result is written once.
+//
+// Backward (vrwkv_rowfuse_bwd; the reference differentiates the PyTorch ops by autograd): with g the gradient of out,
+// z = pre(a), xh = (z - mean) rstd, y = xh w + b (y = z without LayerNorm):
+//   gate:      gy = g sigmoid(o),  g_other = g y sigmoid(o) (1 - sigmoid(o))
+//   residual:  gy = g gamma,       g_other = g (not written: it is g itself),  g_gamma[c] = sum_rows g y
+//   LayerNorm: g_w[c] = sum_rows gy xh,  g_b[c] = sum_rows gy,  gz = rstd (w gy - mean(w gy) - xh mean(w gy xh))
+//   pre:       ga = gz 2 relu(a)  (relu^2)  or  gz
+// A wave walks a run of consecutive rows, recomputes the row statistics from `a`, keeps the per-channel sums of its
+// lanes' channels in registers; the four waves of a workgroup add theirs in LDS and write one partial row per sum,
+// which batch_sum_kernel adds over the workgroups in a fixed order.
 #include "vrwkv_common.h"
 
 namespace vrwkv {
@@ -97,6 +107,219 @@ void rowfuse_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_, co
     }
 }
 
+// Runtime switches (all wave-uniform) instead of template parameters: the backward has many more combinations.
+// SUMS: LayerNorm and / or gamma take part (per-channel vectors and sums in registers); without them the kernel is a
+// plain element-wise pass and rows may be longer.
+template <typename IO, int VPL, bool SUMS>
+__global__ __launch_bounds__(256)
+void rowfuse_bwd_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_, const IO* __restrict__ lnw_,
+                        const IO* __restrict__ lnb_, const IO* __restrict__ gamma_, const IO* __restrict__ g_,
+                        IO* __restrict__ ga_, IO* __restrict__ go_, float* __restrict__ part,
+                        long long rows, int N, float eps, int pre, int post, int rows_per_wave)
+{
+    constexpr int V = 16 / (int)sizeof(IO);
+    extern __shared__ float s_red[];                          // [4 waves][3 sums][N] when channel sums are wanted
+    const bool has_ln = SUMS && lnw_ != nullptr, has_gamma = SUMS && post == POST_RESIDUAL && gamma_ != nullptr;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
+    const int nvec = N / V;
+    constexpr int PV = SUMS ? VPL : 1, PE = SUMS ? V : 1;     // the per-channel arrays exist only with SUMS
+    float w[PV][PE], b[PV][PE], gam[PV][PE], acc_w[PV][PE], acc_b[PV][PE], acc_g[PV][PE];
+#pragma unroll
+    for (int i = 0; i < PV; ++i) {
+        const int vi = lane + WAVE * i;
+        const bool ok = vi < nvec;
+#pragma unroll
+        for (int e = 0; e < PE; ++e) { w[i][e] = 1.f; b[i][e] = 0.f; gam[i][e] = 1.f; acc_w[i][e] = acc_b[i][e] = acc_g[i][e] = 0.f; }
+        if constexpr (SUMS) {
+            if (ok && has_ln) { load_vec<IO, V>(lnw_ + (size_t)vi * V, w[i]); load_vec<IO, V>(lnb_ + (size_t)vi * V, b[i]); }
+            if (ok && has_gamma) load_vec<IO, V>(gamma_ + (size_t)vi * V, gam[i]);
+        }
+    }
+    const long long row0 = ((long long)blockIdx.x * (blockDim.x >> 6) + wave) * rows_per_wave;
+    if constexpr (!SUMS) {
+        // no LayerNorm, no gamma: nothing couples the channels of a row, one vector at a time
+        for (int rr = 0; rr < rows_per_wave; ++rr) {
+            const long long row = row0 + rr;
+            if (row >= rows) break;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int vi = lane + WAVE * i;
+                if (vi >= nvec) continue;
+                const size_t off = (size_t)row * N + (size_t)vi * V;
+                float av[V], gv[V], ov[V], go[V], ga[V];
+                load_vec<IO, V>(a_ + off, av);
+                load_vec<IO, V>(g_ + off, gv);
+                if (post == POST_SIGMOID_GATE) load_vec<IO, V>(other_ + off, ov);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float rl = fmaxf(av[e], 0.f);
+                    const float y = pre == PRE_RELU_SQ ? rl * rl : av[e];
+                    float gy = gv[e];
+                    if (post == POST_SIGMOID_GATE) {
+                        const float sg = fast_rcp(1.f + fast_exp2(-ov[e] * LOG2E));
+                        go[e] = gy * y * sg * (1.f - sg);
+                        gy *= sg;
+                    }
+                    ga[e] = pre == PRE_RELU_SQ ? gy * 2.f * rl : gy;
+                }
+                if (post == POST_SIGMOID_GATE) store_vec<IO, V>(go_ + off, go);
+                store_vec<IO, V>(ga_ + off, ga);
+            }
+        }
+        return;
+    }
+    for (int rr = 0; rr < rows_per_wave; ++rr) {
+        const long long row = row0 + rr;
+        if (row >= rows) break;                               // wave-uniform
+        float r[VPL][V], z[VPL][V], g[VPL][V], o[VPL][V];
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = lane + WAVE * i;
+            if (vi < nvec) {
+                const size_t off = (size_t)row * N + (size_t)vi * V;
+                load_vec<IO, V>(a_ + off, r[i]);
+                load_vec<IO, V>(g_ + off, g[i]);
+                if (post != POST_NONE) load_vec<IO, V>(other_ + off, o[i]);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    if (pre == PRE_RELU_SQ) { r[i][e] = fmaxf(r[i][e], 0.f); z[i][e] = r[i][e] * r[i][e]; }
+                    else z[i][e] = r[i][e];
+                    s += z[i][e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) { r[i][e] = z[i][e] = g[i][e] = o[i][e] = 0.f; }
+            }
+        }
+        float mean = 0.f, rstd = 1.f;
+        if (has_ln) {
+            mean = wave_sum(s) / (float)N;
+            float q = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+                if (lane + WAVE * i < nvec) {
+#pragma unroll
+                    for (int e = 0; e < V; ++e) { const float d = z[i][e] - mean; q = fmaf(d, d, q); }
+                }
+            rstd = rsqrtf(wave_sum(q) / (float)N + eps);
+        }
+        // z becomes xh (normalised) under LayerNorm; g becomes gy
+        float t1 = 0.f, t2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = lane + WAVE * i;
+            if (vi >= nvec) continue;
+            float go[V];
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const int pi = SUMS ? i : 0, pe = SUMS ? e : 0;
+                const float xh = has_ln ? (z[i][e] - mean) * rstd : z[i][e];
+                const float y = has_ln ? fmaf(xh, w[pi][pe], b[pi][pe]) : xh;
+                float gy = g[i][e];
+                if (post == POST_SIGMOID_GATE) {
+                    const float sg = fast_rcp(1.f + fast_exp2(-o[i][e] * LOG2E));
+                    go[e] = gy * y * sg * (1.f - sg);
+                    gy *= sg;
+                } else if (post == POST_RESIDUAL) {
+                    if (has_gamma) { acc_g[pi][pe] = fmaf(gy, y, acc_g[pi][pe]); gy *= gam[pi][pe]; }
+                }
+                if (has_ln) {
+                    acc_b[pi][pe] += gy;
+                    acc_w[pi][pe] = fmaf(gy, xh, acc_w[pi][pe]);
+                    const float t = w[pi][pe] * gy;
+                    t1 += t;
+                    t2 = fmaf(t, xh, t2);
+                    g[i][e] = t;
+                } else {
+                    g[i][e] = gy;
+                }
+                z[i][e] = xh;
+            }
+            if (post == POST_SIGMOID_GATE) store_vec<IO, V>(go_ + (size_t)row * N + (size_t)vi * V, go);
+        }
+        float m1 = 0.f, m2 = 0.f;
+        if (has_ln) { m1 = wave_sum(t1) / (float)N; m2 = wave_sum(t2) / (float)N; }
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = lane + WAVE * i;
+            if (vi >= nvec) continue;
+            float ga[V];
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float gz = has_ln ? rstd * (g[i][e] - m1 - z[i][e] * m2) : g[i][e];
+                ga[e] = pre == PRE_RELU_SQ ? gz * 2.f * r[i][e] : gz;
+            }
+            store_vec<IO, V>(ga_ + (size_t)row * N + (size_t)vi * V, ga);
+        }
+    }
+    if constexpr (SUMS) {
+        // the four waves' channel sums are added in wave order and written as this workgroup's partial rows
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = lane + WAVE * i;
+            if (vi >= nvec) continue;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const int c = vi * V + e;
+                s_red[((size_t)wave * 3 + 0) * N + c] = acc_w[i][e];
+                s_red[((size_t)wave * 3 + 1) * N + c] = acc_b[i][e];
+                s_red[((size_t)wave * 3 + 2) * N + c] = acc_g[i][e];
+            }
+        }
+        __syncthreads();
+        const int nw = blockDim.x >> 6;
+        float* prow = part + (size_t)blockIdx.x * 3 * N;
+        for (int idx = threadIdx.x; idx < 3 * N; idx += blockDim.x) {
+            float sum = 0.f;
+            for (int wv = 0; wv < nw; ++wv) sum += s_red[(size_t)wv * 3 * N + idx];
+            prow[idx] = sum;
+        }
+    }
+}
+
+constexpr int BWD_ROWS_PER_WAVE = 8;
+
+template <typename IO, int VPL, bool SUMS>
+int launch_bwd_vpl(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, const void* g,
+                   void* ga, void* go, float* gparam, float* part, long long rows, int N, int pre, int post, float eps,
+                   hipStream_t st) {
+    const int rows_per_block = 4 * BWD_ROWS_PER_WAVE;
+    const long long nblk = (rows + rows_per_block - 1) / rows_per_block;
+    const size_t lds = SUMS ? (size_t)4 * 3 * N * sizeof(float) : 0;
+    hipLaunchKernelGGL((rowfuse_bwd_kernel<IO, VPL, SUMS>), dim3((unsigned)nblk), dim3(256), lds, st,
+                       static_cast<const IO*>(a), static_cast<const IO*>(other), static_cast<const IO*>(lnw),
+                       static_cast<const IO*>(lnb), static_cast<const IO*>(gamma), static_cast<const IO*>(g),
+                       static_cast<IO*>(ga), static_cast<IO*>(go), part, rows, N, eps, pre, post, BWD_ROWS_PER_WAVE);
+    if (SUMS) {
+        const int wide = 3 * N;                               // gparam: (3, N) = g_weight, g_bias, g_gamma
+        hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gparam,
+                           (const float*)nullptr, (float*)nullptr, (int)nblk, wide);
+    }
+    return check_launch("rowfuse_bwd");
+}
+
+template <typename IO>
+int launch_bwd_io(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, const void* g,
+                  void* ga, void* go, float* gparam, float* part, long long rows, int N, int pre, int post, float eps,
+                  hipStream_t st) {
+    constexpr int V = 16 / (int)sizeof(IO);
+    const int per_lane = (N / V + WAVE - 1) / WAVE;
+    const bool sums = lnw != nullptr || (post == POST_RESIDUAL && gamma != nullptr);
+#define VRWKV_BWD(VPL, SUMS) return launch_bwd_vpl<IO, VPL, SUMS>(a, other, lnw, lnb, gamma, g, ga, go, gparam, part, rows, N, pre, post, eps, st)
+    if (sums) {                                               // at most 16 channels per lane (checked by the caller)
+        if (per_lane <= 1) VRWKV_BWD(1, true);
+        if (per_lane <= 2 || V == 8) VRWKV_BWD(2, true);
+        VRWKV_BWD(4, true);
+    }
+    if (per_lane <= 1) VRWKV_BWD(1, false);
+    if (per_lane <= 2) VRWKV_BWD(2, false);
+    if (per_lane <= 4) VRWKV_BWD(4, false);
+    if (per_lane <= 8) VRWKV_BWD(8, false);
+    VRWKV_BWD(16, false);
+#undef VRWKV_BWD
+}
+
 template <typename IO, int VPL, int PRE, int POST>
 int launch_ln(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
               long long rows, int N, float eps, hipStream_t st) {
@@ -175,6 +398,62 @@ extern "C" int vrwkv_rowfuse(const void* a, const void* other, const void* ln_we
         case VRWKV_F32:  return launch_io<float>(a, other, ln_weight, ln_bias, gamma, out, rows, N, pre, post, eps, st);
         case VRWKV_BF16: return launch_io<__hip_bfloat16>(a, other, ln_weight, ln_bias, gamma, out, rows, N, pre, post, eps, st);
         case VRWKV_F16:  return launch_io<__half>(a, other, ln_weight, ln_bias, gamma, out, rows, N, pre, post, eps, st);
+    }
+    return VRWKV_UNSUPPORTED_DTYPE;
+}
+
+// Channel sums are kept in registers: the backward with LayerNorm or gamma takes rows of at most 16 channels per lane.
+static int rowfuse_bwd_max_n(int) { return 16 * WAVE; }
+
+extern "C" size_t vrwkv_rowfuse_bwd_workspace_bytes(long long rows, int N) {
+    if (rows <= 0 || N <= 0) return 0;
+    const long long nblk = (rows + 4 * BWD_ROWS_PER_WAVE - 1) / (4 * BWD_ROWS_PER_WAVE);
+    return (size_t)nblk * 3 * N * sizeof(float);
+}
+
+extern "C" int vrwkv_rowfuse_bwd(const void* a, const void* other, const void* ln_weight, const void* ln_bias,
+                                 const void* gamma, const void* gout, void* ga, void* gother, float* gparam,
+                                 long long rows, int N, int pre, int post, float eps, int io_dtype,
+                                 void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (rows <= 0 || N <= 0 || pre < 0 || pre > 1 || post < 0 || post > 2) {
+        set_error("rowfuse_bwd: bad arguments (rows=%lld N=%d pre=%d post=%d)", rows, N, pre, post);
+        return VRWKV_INVALID_ARG;
+    }
+    if (io_dtype != VRWKV_F32 && io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16) {
+        set_error("rowfuse_bwd: unsupported io_dtype code %d", io_dtype);
+        return VRWKV_UNSUPPORTED_DTYPE;
+    }
+    const bool sums = ln_weight != nullptr || (post == POST_RESIDUAL && gamma != nullptr);
+    if (!a || !gout || !ga || (post != POST_NONE && !other) || (post == POST_SIGMOID_GATE && !gother) ||
+        ((ln_weight == nullptr) != (ln_bias == nullptr)) || (sums && !gparam)) {
+        set_error("rowfuse_bwd: null pointer argument");
+        return VRWKV_INVALID_ARG;
+    }
+    const int V = io_dtype == VRWKV_F32 ? 4 : 8;
+    if (N % V != 0 || N / V > 16 * WAVE || (sums && N > rowfuse_bwd_max_n(io_dtype)) || rows > 0x7fffffffLL * 32) {
+        set_error("rowfuse_bwd: N=%d must be a multiple of %d, at most %d (%d with LayerNorm or gamma)", N, V,
+                  16 * WAVE * V, rowfuse_bwd_max_n(io_dtype));
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    const uintptr_t all = (uintptr_t)a | (uintptr_t)other | (uintptr_t)ln_weight | (uintptr_t)ln_bias | (uintptr_t)gamma |
+                          (uintptr_t)gout | (uintptr_t)ga | (uintptr_t)gother;
+    if (all & 15) {
+        set_error("rowfuse_bwd: every tensor must be 16-byte aligned");
+        return VRWKV_INVALID_ARG;
+    }
+    if (sums) {
+        const size_t need = vrwkv_rowfuse_bwd_workspace_bytes(rows, N);
+        if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 3)) {
+            set_error("rowfuse_bwd: a 4-byte aligned workspace of %zu bytes is required", need);
+            return VRWKV_WORKSPACE_TOO_SMALL;
+        }
+    }
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    float* part = static_cast<float*>(workspace);
+    switch (io_dtype) {
+        case VRWKV_F32:  return launch_bwd_io<float>(a, other, ln_weight, ln_bias, gamma, gout, ga, gother, gparam, part, rows, N, pre, post, eps, st);
+        case VRWKV_BF16: return launch_bwd_io<__hip_bfloat16>(a, other, ln_weight, ln_bias, gamma, gout, ga, gother, gparam, part, rows, N, pre, post, eps, st);
+        case VRWKV_F16:  return launch_bwd_io<__half>(a, other, ln_weight, ln_bias, gamma, gout, ga, gother, gparam, part, rows, N, pre, post, eps, st);
     }
     return VRWKV_UNSUPPORTED_DTYPE;
 }

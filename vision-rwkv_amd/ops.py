@@ -311,18 +311,79 @@ def row_fuse_tensor_ops(a, other=None, ln_weight=None, ln_bias=None, gamma=None,
     return y
 
 
+class _RowFuse(torch.autograd.Function):
+    """row_fuse with a hand-written backward (vrwkv_rowfuse / vrwkv_rowfuse_bwd).  Per-channel inputs arrive in the
+    dtype of `a` (the casts outside are differentiated by autograd)."""
+
+    @staticmethod
+    def forward(ctx, a, other, ln_weight, ln_bias, gamma, pre, post, eps):
+        ctx.save_for_backward(a, other, ln_weight, ln_bias, gamma)
+        ctx.meta = (pre, post, eps)
+        return _row_fuse_launch(a, other, ln_weight, ln_bias, gamma, pre, post, eps)
+
+    @staticmethod
+    def backward(ctx, gout):
+        a, other, ln_weight, ln_bias, gamma = ctx.saved_tensors
+        pre, post, eps = ctx.meta
+        N = a.shape[-1]
+        rows = a.numel() // N
+        gout = gout.to(a.dtype).contiguous()
+        ga = torch.empty_like(a)
+        go = torch.empty_like(a) if post == POST_SIGMOID_GATE else None
+        sums = ln_weight is not None or (post == POST_RESIDUAL and gamma is not None)
+        L = _lib.lib()
+        gparam = ws = None
+        ws_bytes = 0
+        if sums:
+            gparam = torch.empty(3, N, dtype=torch.float32, device=a.device)
+            ws_bytes = L.vrwkv_rowfuse_bwd_workspace_bytes(rows, N)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        with torch.cuda.device(a.device):
+            _lib.check(L.vrwkv_rowfuse_bwd(a.data_ptr(), ptr(other), ptr(ln_weight), ptr(ln_bias), ptr(gamma),
+                                           gout.data_ptr(), ga.data_ptr(), ptr(go), ptr(gparam), rows, N, pre, post,
+                                           float(eps), _DT[a.dtype], ptr(ws), ws_bytes, _stream_ptr(a.device)))
+        g_other = go if post == POST_SIGMOID_GATE else (gout if post == POST_RESIDUAL else None)
+        g_w = gparam[0].to(ln_weight.dtype) if ln_weight is not None else None
+        g_b = gparam[1].to(ln_bias.dtype) if ln_bias is not None else None
+        g_g = gparam[2].to(gamma.dtype) if (gamma is not None and post == POST_RESIDUAL) else None
+        return ga, g_other, g_w, g_b, g_g, None, None, None
+
+
+def _row_fuse_launch(a, other, ln_weight, ln_bias, gamma, pre, post, eps):
+    out = torch.empty_like(a)
+    N = a.shape[-1]
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().vrwkv_rowfuse(a.data_ptr(), ptr(other), ptr(ln_weight), ptr(ln_bias), ptr(gamma), out.data_ptr(),
+                                            a.numel() // N, N, pre, post, float(eps), _DT[a.dtype], _stream_ptr(a.device)))
+    return out
+
+
 def row_fuse(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NONE, post=POST_NONE, eps=1e-5):
     """One HIP kernel per row-wise epilogue of a block: out = post(LayerNorm(pre(a))) with pre = identity / relu^2,
-    LayerNorm optional, post = identity / sigmoid(other) * y / other + gamma * y.  Forward only: when a gradient is
-    needed, the tensors are not on the GPU, or the row length does not fit, the tensor ops are used instead."""
+    LayerNorm optional, post = identity / sigmoid(other) * y / other + gamma * y; under autograd one backward kernel
+    (rows of at most 1024 channels when LayerNorm or gamma take part).  Where the kernels do not apply (not on the
+    GPU, row length, alignment) the tensor ops are used instead."""
     tensors = [t for t in (a, other, ln_weight, ln_bias, gamma) if t is not None]
     N = a.shape[-1]
     vec = 4 if a.dtype == torch.float32 else 8
+    need_grad = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    sums = ln_weight is not None or (post == POST_RESIDUAL and gamma is not None)
     fits = (ROW_FUSE_ENABLED and a.is_cuda and a.dtype in _DT and N % vec == 0 and N // vec <= 1024 and a.numel() > 0
             and (other is None or (other.shape == a.shape and other.dtype == a.dtype))
-            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
+            and not (need_grad and sums and N > 1024))
     if not fits:
         return row_fuse_tensor_ops(a, other, ln_weight, ln_bias, gamma, pre, post, eps)
+    if need_grad:
+        ac = a.contiguous()
+        oc = other.contiguous() if other is not None else None
+        par = [p.reshape(-1).to(a.dtype).contiguous() if p is not None else None for p in (ln_weight, ln_bias, gamma)]
+        if post != POST_RESIDUAL:
+            par[2] = None
+        if not _vec_ok(ac, oc, *par) or any(p is not None and p.numel() != N for p in par):
+            return row_fuse_tensor_ops(a, other, ln_weight, ln_bias, gamma, pre, post, eps)
+        return _RowFuse.apply(ac, oc, par[0], par[1], par[2], pre, post, float(eps))
     a = a.contiguous()
     other = other.contiguous() if other is not None else None
     par = [p.detach().reshape(-1).to(a.dtype).contiguous() if p is not None else None for p in (ln_weight, ln_bias, gamma)]
@@ -331,12 +392,7 @@ def row_fuse(a, other=None, ln_weight=None, ln_bias=None, gamma=None, pre=PRE_NO
     for p in par:
         if p is not None and p.numel() != N:
             raise RuntimeError("LayerNorm weight, bias and gamma must have one element per channel")
-    out = torch.empty_like(a)
-    ptr = lambda t: t.data_ptr() if t is not None else None
-    with torch.cuda.device(a.device):
-        _lib.check(_lib.lib().vrwkv_rowfuse(a.data_ptr(), ptr(other), ptr(par[0]), ptr(par[1]), ptr(par[2]), out.data_ptr(),
-                                            a.numel() // N, N, pre, post, float(eps), _DT[a.dtype], _stream_ptr(a.device)))
-    return out
+    return _row_fuse_launch(a, other, par[0], par[1], par[2], pre, post, eps)
 
 
 def maa_mix_tensor_ops(x, sx, m, maas):
