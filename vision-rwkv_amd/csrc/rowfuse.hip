@@ -278,19 +278,21 @@ void rowfuse_bwd_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_
     }
 }
 
-constexpr int BWD_ROWS_PER_WAVE = 8;
+constexpr int BWD_ROWS_PER_WAVE = 8;      // with channel sums: one partial row per 32 rows
+constexpr int BWD_ROWS_PER_WAVE_PLAIN = 2;   // element-wise only: more workgroups in flight
 
 template <typename IO, int VPL, bool SUMS>
 int launch_bwd_vpl(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, const void* g,
                    void* ga, void* go, float* gparam, float* part, long long rows, int N, int pre, int post, float eps,
                    hipStream_t st) {
-    const int rows_per_block = 4 * BWD_ROWS_PER_WAVE;
+    const int rpw = SUMS ? BWD_ROWS_PER_WAVE : BWD_ROWS_PER_WAVE_PLAIN;
+    const int rows_per_block = 4 * rpw;
     const long long nblk = (rows + rows_per_block - 1) / rows_per_block;
     const size_t lds = SUMS ? (size_t)4 * 3 * N * sizeof(float) : 0;
     hipLaunchKernelGGL((rowfuse_bwd_kernel<IO, VPL, SUMS>), dim3((unsigned)nblk), dim3(256), lds, st,
                        static_cast<const IO*>(a), static_cast<const IO*>(other), static_cast<const IO*>(lnw),
                        static_cast<const IO*>(lnb), static_cast<const IO*>(gamma), static_cast<const IO*>(g),
-                       static_cast<IO*>(ga), static_cast<IO*>(go), part, rows, N, eps, pre, post, BWD_ROWS_PER_WAVE);
+                       static_cast<IO*>(ga), static_cast<IO*>(go), part, rows, N, eps, pre, post, rpw);
     if (SUMS) {
         const int wide = 3 * N;                               // gparam: (3, N) = g_weight, g_bias, g_gamma
         hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gparam,
