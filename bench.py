@@ -229,6 +229,16 @@ def backbone_section(torch, ops, steps, warmup):
         netb(imgb).float().square().mean().backward()
 
     ms_train = timed(train_step, max(steps // 2, 3), max(warmup // 4, 3))
+    del netb
+    net6t = ops.vrwkv6_b().to(dev).bfloat16()
+    net6t.train()
+
+    def train_step6():
+        net6t.zero_grad(set_to_none=True)
+        net6t(imgb).float().square().mean().backward()
+
+    ms_train6 = timed(train_step6, max(steps // 2, 3), max(warmup // 4, 3))
+    del net6t
     return {"workload": f"VRWKV-L forward, batch {Bn}, {S}x{S}, T={Tn}, C={Cn}, 24 blocks, bf16, random weights",
             "ms_per_forward": round(ms_fwd, 3), "images_per_s": round(Bn / ms_fwd * 1e3, 1),
             "ms_per_forward_unfused_shift": round(ms_fwd_eager_shift, 3),
@@ -237,6 +247,9 @@ def backbone_section(torch, ops, steps, warmup):
             "vrwkv_b_train": {"workload": "VRWKV-B forward + backward (no optimizer step), batch 64, 224x224, T=196, C=768, "
                                           "12 blocks, bf16, random weights, Bi-WKV forward and backward on the HIP kernels",
                               "ms_per_step": round(ms_train, 3), "images_per_s": round(64 / ms_train * 1e3, 1)},
+            "vrwkv6_b_train": {"workload": "VRWKV6-B forward + backward (no optimizer step), batch 64, 224x224, T=196, C=768, "
+                                           "12 heads, 12 blocks, bf16, random weights, wkv6 forward and backward on the HIP kernels",
+                               "ms_per_step": round(ms_train6, 3), "images_per_s": round(64 / ms_train6 * 1e3, 1)},
             "vrwkv6_b": {"workload": "VRWKV6-B forward, batch 64, 224x224, T=196, C=768, 12 heads, 12 blocks, bf16, "
                                      "random weights",
                          "ms_per_forward": round(ms6, 3), "images_per_s": round(B6 / ms6 * 1e3, 1),

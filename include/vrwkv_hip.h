@@ -152,6 +152,21 @@ int vrwkv_maa_mix(const void* x, const void* sx, const void* m, const float* maa
 int vrwkv_groupnorm_gate(const void* y, const void* gate, const void* gn_weight, const void* gn_bias, void* out,
                          long long rows, int C, int group, float eps, int y_dtype, int io_dtype, void* hip_stream);
 
+/* Backward of the two (the reference differentiates its PyTorch ops by autograd; no native code).
+ * vrwkv_maa_mix_bwd: gout[i] gradients of out[i]; gx, gsx: (rows, C), gm: (5, rows, C) of io_dtype; gmaa: (5, C) fp32
+ *   summed over the rows in a fixed order; workspace vrwkv_maa_mix_bwd_workspace_bytes(rows, C) bytes.
+ * vrwkv_groupnorm_gate_bwd: gout gradient of out (io_dtype); gy in y's type, ggate in io_dtype; gparam: (2, C) fp32 =
+ *   gradients of gn_weight and gn_bias; C at most 1024; workspace vrwkv_groupnorm_gate_bwd_workspace_bytes(rows, C). */
+size_t vrwkv_maa_mix_bwd_workspace_bytes(long long rows, int C);
+int vrwkv_maa_mix_bwd(const void* x, const void* sx, const void* m, const float* maa, const void* const* gout,
+                      void* gx, void* gsx, void* gm, float* gmaa, long long rows, int C, int io_dtype,
+                      void* workspace, size_t workspace_bytes, void* hip_stream);
+size_t vrwkv_groupnorm_gate_bwd_workspace_bytes(long long rows, int C);
+int vrwkv_groupnorm_gate_bwd(const void* y, const void* gate, const void* gn_weight, const void* gn_bias,
+                             const void* gout, void* gy, void* ggate, float* gparam, long long rows, int C, int group,
+                             float eps, int y_dtype, int io_dtype, void* workspace, size_t workspace_bytes,
+                             void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -353,3 +353,59 @@ def test_row_fuse_backward_against_autograd(N, dtype, with_sums):
             assert t.grad is not None, (name, pre, post, ln)
             err = (t.grad.double() - r.grad).abs().max().item() / max(r.grad.abs().max().item(), 1e-6)
             assert err <= tol, (name, pre, post, ln, use_gamma, err)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,T,C,dtype", [(2, 5, 64, torch.float32), (3, 37, 768, torch.float32), (2, 23, 768, torch.bfloat16),
+                                          (1, 7, 128, torch.float16)])
+def test_vrwkv6_mix_backward_against_autograd(B, T, C, dtype):
+    """Gradients of maa_mix and groupnorm_gate (hand-written backward kernels) against autograd through the tensor-op
+    sequences in float64 on the same inputs; row counts that leave the last workgroup partial.
+    Tolerance: 1e-4 of each gradient's scale for fp32 I/O, 3e-2 for 16-bit."""
+    import vision_rwkv_amd as ops
+    O = ops.ops
+    dev = "cuda:0"
+    torch.manual_seed(C + T)
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    d = lambda t: t.detach().double().requires_grad_(True)
+
+    def check(name, got, ref):
+        err = (got.double() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-6)
+        assert err <= tol, (name, err)
+
+    x = torch.randn(B, T, C, device=dev).to(dtype).requires_grad_(True)
+    sx = torch.randn(B, T, C, device=dev).to(dtype).requires_grad_(True)
+    m = (0.3 * torch.randn(5, B, T, C, device=dev)).to(dtype).requires_grad_(True)
+    maas = [torch.rand(1, 1, C, device=dev).to(dtype).requires_grad_(True) for _ in range(5)]
+    gouts = [torch.randn(B, T, C, device=dev).to(dtype) for _ in range(5)]
+    outs = ops.maa_mix(x, sx, m, maas)
+    assert "MaaMix" in type(outs[0].grad_fn).__name__
+    torch.autograd.backward(outs, gouts)
+    x2, sx2, m2, maas2 = d(x), d(sx), d(m), [d(a) for a in maas]
+    ref = O.maa_mix_tensor_ops(x2, sx2, m2, maas2)
+    torch.autograd.backward(ref, [g.double() for g in gouts])
+    for o, r in zip(outs, ref):
+        check("out", o, r.detach())
+    check("gx", x.grad, x2.grad); check("gsx", sx.grad, sx2.grad); check("gm", m.grad, m2.grad)
+    for a, a2 in zip(maas, maas2):
+        assert a.grad.shape == a.shape
+        check("gmaa", a.grad, a2.grad)
+
+    if dtype != torch.float32:
+        H = C // 64
+        for ydt in (torch.float32, dtype):
+            y = (3 * torch.randn(B, T, C, device=dev) + 1).to(ydt).requires_grad_(True)
+            gate = torch.randn(B, T, C, device=dev).to(dtype).requires_grad_(True)
+            w = (1 + 0.3 * torch.randn(C, device=dev)).to(dtype).requires_grad_(True)
+            b = (0.3 * torch.randn(C, device=dev)).to(dtype).requires_grad_(True)
+            gout = torch.randn(B, T, C, device=dev).to(dtype)
+            out = ops.groupnorm_gate(y, gate, w, b, H)
+            assert "GroupNormGate" in type(out.grad_fn).__name__
+            out.backward(gout)
+            y2, g2, w2, b2 = d(y), d(gate), d(w), d(b)
+            ref = O.groupnorm_gate_tensor_ops(y2, g2, w2, b2, H)
+            ref.backward(gout.double())
+            check("out", out, ref.detach())
+            assert y.grad.dtype == ydt
+            check("gy", y.grad, y2.grad); check("ggate", gate.grad, g2.grad)
+            check("gw", w.grad, w2.grad); check("gb", b.grad, b2.grad)

@@ -75,6 +75,14 @@ def _declare(lib):
     lib.vrwkv_maa_mix.restype = i
     lib.vrwkv_groupnorm_gate.argtypes = [vp, vp, vp, vp, vp, c.c_longlong, i, i, c.c_float, i, i, vp]
     lib.vrwkv_groupnorm_gate.restype = i
+    lib.vrwkv_maa_mix_bwd_workspace_bytes.argtypes = [c.c_longlong, i]
+    lib.vrwkv_maa_mix_bwd_workspace_bytes.restype = sz
+    lib.vrwkv_maa_mix_bwd.argtypes = [vp, vp, vp, fp, c.POINTER(c.c_void_p), vp, vp, vp, fp, c.c_longlong, i, i, vp, sz, vp]
+    lib.vrwkv_maa_mix_bwd.restype = i
+    lib.vrwkv_groupnorm_gate_bwd_workspace_bytes.argtypes = [c.c_longlong, i]
+    lib.vrwkv_groupnorm_gate_bwd_workspace_bytes.restype = sz
+    lib.vrwkv_groupnorm_gate_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, fp, c.c_longlong, i, i, c.c_float, i, i, vp, sz, vp]
+    lib.vrwkv_groupnorm_gate_bwd.restype = i
     return lib
 
 

@@ -401,30 +401,67 @@ def maa_mix_tensor_ops(x, sx, m, maas):
     return [x + xx * (maa + mi) for maa, mi in zip(maas, m.unbind(0))]
 
 
-def maa_mix(x, sx, m, maas, maa_table=None):
-    """The five data-dependent token mixes of VRWKV6 (vrwkv6.py:190-194) in one HIP kernel: x, sx (the shifted x):
-    (B,T,C); m: (5,B,T,C); maas: the five (C,) vectors time_maa_w, _k, _v, _r, _g (or their stacked fp32 table).
-    Forward only: tensor ops under autograd or when the kernel does not apply."""
+class _MaaMix(torch.autograd.Function):
+    """maa_mix with a hand-written backward (vrwkv_maa_mix / vrwkv_maa_mix_bwd); the five vectors enter as one (5, C)
+    fp32 table built by differentiable tensor ops outside."""
+
+    @staticmethod
+    def forward(ctx, x, sx, m, table):
+        ctx.save_for_backward(x, sx, m, table)
+        return tuple(_maa_mix_launch(x, sx, m, table))
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        x, sx, m, table = ctx.saved_tensors
+        C = x.shape[-1]
+        rows = x.numel() // C
+        gs = [g.to(x.dtype).contiguous() for g in gouts]
+        gx, gsx, gm = torch.empty_like(x), torch.empty_like(x), torch.empty_like(m)
+        gmaa = torch.empty_like(table)
+        L = _lib.lib()
+        ws_bytes = L.vrwkv_maa_mix_bwd_workspace_bytes(rows, C)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        ptrs = (ctypes.c_void_p * 5)(*[g.data_ptr() for g in gs])
+        with torch.cuda.device(x.device):
+            _lib.check(L.vrwkv_maa_mix_bwd(x.data_ptr(), sx.data_ptr(), m.data_ptr(), table.data_ptr(), ptrs, gx.data_ptr(),
+                                           gsx.data_ptr(), gm.data_ptr(), gmaa.data_ptr(), rows, C, _DT[x.dtype],
+                                           ws.data_ptr(), ws_bytes, _stream_ptr(x.device)))
+        return gx, gsx, gm, gmaa
+
+
+def _maa_mix_launch(x, sx, m, table):
     C = x.shape[-1]
-    vec = 4 if x.dtype == torch.float32 else 8
-    tensors = [x, sx, m] + list(maas)
-    fits = (ROW_FUSE_ENABLED and x.is_cuda and x.dtype in _DT and C % vec == 0 and x.numel() > 0
-            and sx.shape == x.shape and sx.dtype == x.dtype and m.dtype == x.dtype and tuple(m.shape) == (5,) + tuple(x.shape)
-            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
-    if not fits:
-        return maa_mix_tensor_ops(x, sx, m, maas)
-    x, sx, m = x.contiguous(), sx.contiguous(), m.contiguous()
-    if not _vec_ok(x, sx, m):
-        return maa_mix_tensor_ops(x, sx, m, maas)
-    table = maa_table if maa_table is not None else stack_mixes(maas, x.device)
-    if tuple(table.shape) != (5, C) or table.dtype != torch.float32 or not table.is_contiguous():
-        raise RuntimeError("maa table must be a contiguous float32 (5, C) tensor")
     outs = [torch.empty_like(x) for _ in range(5)]
     ptrs = (ctypes.c_void_p * 5)(*[o.data_ptr() for o in outs])
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().vrwkv_maa_mix(x.data_ptr(), sx.data_ptr(), m.data_ptr(), table.data_ptr(), ptrs,
                                             x.numel() // C, C, _DT[x.dtype], _stream_ptr(x.device)))
     return outs
+
+
+def maa_mix(x, sx, m, maas, maa_table=None):
+    """The five data-dependent token mixes of VRWKV6 (vrwkv6.py:190-194) in one HIP kernel: x, sx (the shifted x):
+    (B,T,C); m: (5,B,T,C); maas: the five (C,) vectors time_maa_w, _k, _v, _r, _g (or their stacked fp32 table).
+    Under autograd one backward kernel; tensor ops when the kernels do not apply."""
+    C = x.shape[-1]
+    vec = 4 if x.dtype == torch.float32 else 8
+    tensors = [x, sx, m] + list(maas)
+    need_grad = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    fits = (ROW_FUSE_ENABLED and x.is_cuda and x.dtype in _DT and C % vec == 0 and x.numel() > 0
+            and sx.shape == x.shape and sx.dtype == x.dtype and m.dtype == x.dtype and tuple(m.shape) == (5,) + tuple(x.shape)
+            and not (need_grad and x.numel() // C > 65535 * 32))
+    if not fits:
+        return maa_mix_tensor_ops(x, sx, m, maas)
+    xc, sxc, mc = x.contiguous(), sx.contiguous(), m.contiguous()
+    if not _vec_ok(xc, sxc, mc):
+        return maa_mix_tensor_ops(x, sx, m, maas)
+    if need_grad:
+        table = torch.stack([a.reshape(-1).float() for a in maas])      # differentiable: the vectors' gradients flow through it
+        return list(_MaaMix.apply(xc, sxc, mc, table))
+    table = maa_table if maa_table is not None else stack_mixes(maas, x.device)
+    if tuple(table.shape) != (5, C) or table.dtype != torch.float32 or not table.is_contiguous():
+        raise RuntimeError("maa table must be a contiguous float32 (5, C) tensor")
+    return _maa_mix_launch(xc, sxc, mc, table)
 
 
 def groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
@@ -434,28 +471,67 @@ def groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
     return yn.view(gate.shape) * torch.nn.functional.silu(gate)
 
 
-def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
-    """GroupNorm(n_groups, C) of every token of y (fp32 as RUN_CUDA_RWKV6 returns it, or gate's dtype) times
-    silu(gate), in one HIP kernel (vrwkv6.py:199, 205-211).  Forward only, 16-bit gate / output; tensor ops otherwise."""
+class _GroupNormGate(torch.autograd.Function):
+    """groupnorm_gate with a hand-written backward (vrwkv_groupnorm_gate / vrwkv_groupnorm_gate_bwd)."""
+
+    @staticmethod
+    def forward(ctx, y, gate, w, b, group, eps):
+        ctx.save_for_backward(y, gate, w, b)
+        ctx.meta = (group, eps)
+        return _groupnorm_gate_launch(y, gate, w, b, group, eps)
+
+    @staticmethod
+    def backward(ctx, gout):
+        y, gate, w, b = ctx.saved_tensors
+        group, eps = ctx.meta
+        C = y.shape[-1]
+        rows = y.numel() // C
+        gout = gout.to(gate.dtype).contiguous()
+        gy, gg = torch.empty_like(y), torch.empty_like(gate)
+        gparam = torch.empty(2, C, dtype=torch.float32, device=y.device)
+        L = _lib.lib()
+        ws_bytes = L.vrwkv_groupnorm_gate_bwd_workspace_bytes(rows, C)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=y.device)
+        with torch.cuda.device(y.device):
+            _lib.check(L.vrwkv_groupnorm_gate_bwd(y.data_ptr(), gate.data_ptr(), w.data_ptr(), b.data_ptr(), gout.data_ptr(),
+                                                  gy.data_ptr(), gg.data_ptr(), gparam.data_ptr(), rows, C, group, float(eps),
+                                                  _DT[y.dtype], _DT[gate.dtype], ws.data_ptr(), ws_bytes, _stream_ptr(y.device)))
+        return gy, gg, gparam[0].to(w.dtype), gparam[1].to(b.dtype), None, None
+
+
+def _groupnorm_gate_launch(y, gate, w, b, group, eps):
     C = y.shape[-1]
-    group = C // n_groups if n_groups > 0 and C % n_groups == 0 else 0
-    tensors = [y, gate, gn_weight, gn_bias]
-    fits = (ROW_FUSE_ENABLED and y.is_cuda and gate.dtype in (torch.bfloat16, torch.float16) and y.shape == gate.shape
-            and y.dtype in (torch.float32, gate.dtype) and group in (8, 16, 32, 64, 128) and y.numel() > 0
-            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)))
-    if not fits:
-        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
-    y, gate = y.contiguous(), gate.contiguous()
-    w = gn_weight.detach().to(gate.dtype).contiguous()
-    b = gn_bias.detach().to(gate.dtype).contiguous()
-    if not _vec_ok(y, gate, w, b):
-        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
     out = torch.empty_like(gate)
     with torch.cuda.device(y.device):
         _lib.check(_lib.lib().vrwkv_groupnorm_gate(y.data_ptr(), gate.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(),
                                                    y.numel() // C, C, group, float(eps), _DT[y.dtype], _DT[gate.dtype],
                                                    _stream_ptr(y.device)))
     return out
+
+
+def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
+    """GroupNorm(n_groups, C) of every token of y (fp32 as RUN_CUDA_RWKV6 returns it, or gate's dtype) times
+    silu(gate), in one HIP kernel (vrwkv6.py:199, 205-211), and one backward kernel under autograd (C <= 1024);
+    16-bit gate / output; tensor ops otherwise."""
+    C = y.shape[-1]
+    group = C // n_groups if n_groups > 0 and C % n_groups == 0 else 0
+    tensors = [y, gate, gn_weight, gn_bias]
+    need_grad = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    fits = (ROW_FUSE_ENABLED and y.is_cuda and gate.dtype in (torch.bfloat16, torch.float16) and y.shape == gate.shape
+            and y.dtype in (torch.float32, gate.dtype) and group in (8, 16, 32, 64, 128) and y.numel() > 0
+            and not (need_grad and C > 1024))
+    if not fits:
+        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
+    yc, gc = y.contiguous(), gate.contiguous()
+    if need_grad:
+        w, b = gn_weight.to(gate.dtype).contiguous(), gn_bias.to(gate.dtype).contiguous()
+    else:
+        w, b = gn_weight.detach().to(gate.dtype).contiguous(), gn_bias.detach().to(gate.dtype).contiguous()
+    if not _vec_ok(yc, gc, w, b):
+        return groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps)
+    if need_grad:
+        return _GroupNormGate.apply(yc, gc, w, b, group, float(eps))
+    return _groupnorm_gate_launch(yc, gc, w, b, group, eps)
 
 
 class _QShiftMix(torch.autograd.Function):
