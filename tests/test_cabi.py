@@ -97,6 +97,21 @@ def test_elementwise_entry_points_validate_without_device(lib):
     assert gg(one, one, one, one, one, 4, 128, 48, 1e-5, 0, 1, None) == 3                      # C not a multiple of the group
     assert gg(one, one, one, one, one, 4, 96, 24, 1e-5, 0, 1, None) == 3                       # group not 8..128 in powers of two
     assert b"group" in lib.vrwkv_last_error()
+    mb = lib.vrwkv_maa_mix_bwd
+    gouts = (ctypes.c_void_p * 5)(64, 64, 64, 64, 64)
+    assert lib.vrwkv_maa_mix_bwd_workspace_bytes(100, 768) == 4 * 5 * 768 * 4                 # one partial row set per 32 rows
+    assert mb(one, one, one, one, gouts, one, one, one, None, 4, 64, 1, None, 0, None) == 1    # gmaa is null
+    assert mb(one, one, one, one, gouts, one, one, one, one, 4, 64, 5, None, 0, None) == 2     # unknown dtype
+    assert mb(one, one, one, one, gouts, one, one, one, one, 4, 60, 1, None, 0, None) == 3     # C not a multiple of 8
+    assert mb(one, one, one, one, gouts, one, one, one, one, 4, 64, 1, None, 0, None) == 5     # workspace missing
+    gouts[2] = None
+    assert mb(one, one, one, one, gouts, one, one, one, one, 4, 64, 1, one, 1 << 20, None) == 1   # a null gradient
+    gb = lib.vrwkv_groupnorm_gate_bwd
+    assert lib.vrwkv_groupnorm_gate_bwd_workspace_bytes(100, 768) == 4 * 2 * 768 * 4          # one partial row pair per 32 rows
+    assert gb(one, one, one, one, one, one, one, None, 4, 128, 64, 1e-5, 0, 1, None, 0, None) == 1    # gparam is null
+    assert gb(one, one, one, one, one, one, one, one, 4, 128, 64, 1e-5, 0, 0, None, 0, None) == 2     # fp32 gate
+    assert gb(one, one, one, one, one, one, one, one, 4, 2048, 64, 1e-5, 0, 1, None, 0, None) == 3    # more than 1024 channels
+    assert gb(one, one, one, one, one, one, one, one, 4, 128, 64, 1e-5, 0, 1, None, 0, None) == 5     # workspace missing
 
 
 def test_python_boundary_errors_without_device():
