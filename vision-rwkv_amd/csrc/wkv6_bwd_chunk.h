@@ -110,15 +110,32 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
     f32x16 S0 = {0}, S1 = {0};      // state tiles: rows c = 32*ch2 + 8(r/4)+4g+(r%4), column o = ocol
     float xcarry = 0.f, gu_acc = 0.f;   // GK: sum of (a - b) over the tokens scanned so far; GR: gu
     RawW wraw[16];
+    // Row offsets walk the 16 tokens of this wave's block with one scalar add each; rows past T (last chunk only)
+    // are clamped to the last row and switched off where they are used.
+    const int sgn = ASC ? 1 : -1;
     auto fetch_w = [&](int ch, int C) {
-        const int c = chunk_of(ch);
+        const unsigned step = (unsigned)(sgn * C * (int)sizeof(WT)), last = (unsigned)(T - 1) * C * (unsigned)sizeof(WT);
+        unsigned so = (unsigned)token_of_n(chunk_of(ch), 16 * q) * C * (unsigned)sizeof(WT);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const int t = token_of_n(c, 16 * q + m);
-            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(WT));
+            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), so < last ? so : last);
+            so += step;
         }
     };
     fetch_w(0, C);
+    // causal masks of the in-chunk matrix, one word per pair of accumulator registers (r = 2p low half, 2p + 1 high):
+    // the lane holds column t = x and rows s = 8(r/4) + 4g + (r%4).  The GK scans have no registers to spare for
+    // them and mask with compares instead.
+    constexpr bool MASK_REGS = KIND != SCAN_GK;
+    unsigned keepw[8], diagw[8];
+    if (MASK_REGS) {
+#pragma unroll
+        for (int pr = 0; pr < 8; ++pr) {
+            const int s0 = 8 * ((2 * pr) / 4) + 4 * g + ((2 * pr) % 4);
+            keepw[pr] = (s0 < x ? 0xffffu : 0u) | (s0 + 1 < x ? 0xffff0000u : 0u);
+            diagw[pr] = (s0 == x ? 0xffffu : 0u) | (s0 + 1 == x ? 0xffff0000u : 0u);
+        }
+    }
 
     for (int ch = 0; ch < nchunk; ++ch) {
         int Cs = C;
@@ -129,80 +146,119 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
         // wave q prepares pass indices n = 16q .. 16q+15 of the chunk; lane = channel
         RawIO xraw[16], yraw[16];                          // the two bf16 tensors this scan needs here
         unsigned graw[16];                                 // gy (fp32 bits)
+        {
+            const unsigned last = (unsigned)(T - 1) * Cs;
+            unsigned so = (unsigned)token_of_n(cc, 16 * q) * Cs;          // element offset of the row
+            const unsigned step = (unsigned)(sgn * Cs);
 #pragma unroll
-        for (int m = 0; m < 16; ++m) {
-            const int t = token_of_n(cc, 16 * q + m);
-            const unsigned tt = (unsigned)(t < T ? t : 0);
-            const unsigned so = tt * Cs * 2u, vo = lane * 2u;
-            if (KIND == SCAN_GR) { xraw[m] = BufRaw<2>::ld(rsv, vo, so); yraw[m] = BufRaw<2>::ld(rsk, vo, so); }
-            if (KIND == SCAN_GK) { xraw[m] = BufRaw<2>::ld(rsv, vo, so); yraw[m] = BufRaw<2>::ld(rsr, vo, so); }
-            if (KIND == SCAN_GV) { xraw[m] = BufRaw<2>::ld(rsk, vo, so); yraw[m] = BufRaw<2>::ld(rsr, vo, so); }
-            graw[m] = BufRaw<4>::ld(rsg, lane * 4u, tt * Cs * 4u);
+            for (int m = 0; m < 16; ++m) {
+                const unsigned sc = so < last ? so : last;
+                const unsigned vo = lane * 2u;
+                if (KIND == SCAN_GR) { xraw[m] = BufRaw<2>::ld(rsv, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsk, vo, sc * 2u); }
+                if (KIND == SCAN_GK) { xraw[m] = BufRaw<2>::ld(rsv, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsr, vo, sc * 2u); }
+                if (KIND == SCAN_GV) { xraw[m] = BufRaw<2>::ld(rsk, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsr, vo, sc * 2u); }
+                graw[m] = BufRaw<4>::ld(rsg, lane * 4u, sc * 4u);
+                so += step;
+            }
         }
-        float ld[16];
-#pragma unroll
-        for (int m = 0; m < 16; ++m) {
-            const bool ok = token_of_n(cc, 16 * q + m) < T;
-            const float fw = cvtw(wraw[m]);
-            ld[m] = ok ? (W_IS_EW ? fw : -__expf(fw)) : 0.f;
-        }
+        // log decays in log2 units: ld2 = -log2(e) exp(w) = -exp2(w log2(e) + log2(log2(e)))
+        const bool full = (cc + 1) * LC <= T;                             // wave-uniform: no token of the chunk is past T
         float p[16];
-        p[0] = ld[0];
+        {
+            float e[16];
 #pragma unroll
-        for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
+            for (int m = 0; m < 16; ++m) {
+                const float fw = cvtw(wraw[m]);
+                e[m] = W_IS_EW ? -fw * LOG2E : fast_exp2(fmaf(fw, LOG2E, LOG2_LOG2E));
+            }
+            if (!full) {
+#pragma unroll
+                for (int m = 0; m < 16; ++m)
+                    if (token_of_n(cc, 16 * q + m) >= T) e[m] = 0.f;
+            }
+            p[0] = -e[0];
+#pragma unroll
+            for (int m = 1; m < 16; ++m) p[m] = p[m - 1] - e[m];
+        }
         if (q == 0) L.Tot[lane] = p[15];
         WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
         WKV6_STAMP(2);
-        const float pref = L.Tot[lane];                                  // P_15
-        const float off = q == 1 ? pref : 0.f;
+        const float pref = L.Tot[lane];                                  // P_15 (log2 units)
+        const float dq = q == 1 ? 0.f : -pref;                           // z_m = P_m - Pref = p[m] + dq
         if (q == 1) {
-            const float p31 = p[15] + off;
-            L.C2[lane] = __expf(p31);
-            L.C3[lane] = __expf(p31 - pref);
-            if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY)) != 0ull && lane == 0) sFlag = 1;
+            const float p31 = p[15] + pref;
+            L.C2[lane] = fast_exp2(p31);
+            L.C3[lane] = fast_exp2(p[15]);
+            if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag = 1;
         } else {
-            L.C1[lane] = __expf(pref);
+            L.C1[lane] = fast_exp2(pref);
         }
         {
-            bf16x8 kth[2], ktl[2], vth[2], vtl[2];
+            if (!full) {
+                // a token past T is switched off through the one operand every product of this scan contains
+                // (k for GR, r for GK and GV); its own output rows are dropped by the stores
+#pragma unroll
+                for (int m = 0; m < 16; ++m)
+                    if (token_of_n(cc, 16 * q + m) >= T) yraw[m] = RawIO{};
+            }
+            unsigned kthw[8], ktlw[8], vthw[8], vtlw[8];
             float pu[16];
             const int r0 = REV ? 16 * (1 - q) : 16 * q;                   // first scan row of this wave's block
+            float zp = dq;                                                // Pex_m - Pref = z_(m-1)
 #pragma unroll
-            for (int m = 0; m < 16; ++m) {
-                const int n = 16 * q + m;
-                const int e = REV ? 15 - m : m;                           // position inside this wave's 16 scan rows
-                const int rho = r0 + e;                                   // = n, or 31 - n for a reversed scan
-                const bool ok = token_of_n(cc, n) < T;
-                const float P = p[m] + off;
-                const float f1 = __expf((m ? p[m - 1] : 0.f) + off - pref);  // exp(Pex - Pref), Pex_m = P_(m-1)
-                const float f2 = __expf(pref - P);                        // exp(Pref - P)
-                const float xa = ok ? cvt(xraw[m]) : 0.f, ya = ok ? cvt(yraw[m]) : 0.f;
-                const float gyv = ok ? __builtin_bit_cast(float, graw[m]) : 0.f;
-                // per scan: Q value, Kc value, Val value of this (token, channel)
-                float qv, kcv, valv;
-                if (KIND == SCAN_GR) { qv = gyv; kcv = xa; valv = ya * f2; L.Post[rho][lane] = f1; }
-                if (KIND == SCAN_GK) { qv = xa; kcv = gyv; valv = ya * f1; L.Post[rho][lane] = f2; }
-                if (KIND == SCAN_GV) { qv = xa * f2; kcv = ya * f1; valv = gyv; pu[m] = ya * u_e * xa; }
-                const __bf16 qh = (__bf16)qv, kh = (__bf16)kcv, vh = (__bf16)valv;
-                L.Qh[rho][lane] = qh;
-                if (QS) L.Ql[rho][lane] = (__bf16)(qv - (float)qh);
-                L.Kh[rho][lane] = kh;
-                kth[e >> 3][e & 7] = kh;
-                if (KS) {
-                    const __bf16 kl = (__bf16)(kcv - (float)kh);
-                    L.Kl[rho][lane] = kl;
-                    ktl[e >> 3][e & 7] = kl;
+            for (int m = 0; m < 16; m += 2) {
+                const float z0 = p[m] + dq, z1 = p[m + 1] + dq;
+                const float f1a = fast_exp2(zp), f2a = fast_exp2(-z0);    // exp(Pex - Pref), exp(Pref - P)
+                const float f1b = fast_exp2(z0), f2b = fast_exp2(-z1);
+                zp = z1;
+                // tokens (lo, hi) of a packed word: scan rows rho_lo (even position e) and rho_lo + 1
+                const int e_lo = REV ? 14 - m : m;                        // position inside this wave's 16 scan rows
+                const int rho_lo = r0 + e_lo, rho_hi = rho_lo + 1;
+                const int m_lo = REV ? m + 1 : m, m_hi = REV ? m : m + 1;
+                const float f1_lo = REV ? f1b : f1a, f1_hi = REV ? f1a : f1b;
+                const float f2_lo = REV ? f2b : f2a, f2_hi = REV ? f2a : f2b;
+                const float xa_lo = cvt(xraw[m_lo]), xa_hi = cvt(xraw[m_hi]);
+                const float ya_lo = cvt(yraw[m_lo]), ya_hi = cvt(yraw[m_hi]);
+                const float gy_lo = __builtin_bit_cast(float, graw[m_lo]), gy_hi = __builtin_bit_cast(float, graw[m_hi]);
+                const unsigned xbits = (unsigned)xraw[m_lo] | ((unsigned)xraw[m_hi] << 16);   // bf16 pair as loaded
+                // per scan: Q, Kc, Val of this (token, channel); exact bf16 inputs keep their bits
+                float q_lo, q_hi, k_lo, k_hi, v_lo, v_hi;
+                if (KIND == SCAN_GR) { q_lo = gy_lo; q_hi = gy_hi; v_lo = ya_lo * f2_lo; v_hi = ya_hi * f2_hi;
+                                       L.Post[rho_lo][lane] = f1_lo; L.Post[rho_hi][lane] = f1_hi; }
+                if (KIND == SCAN_GK) { k_lo = gy_lo; k_hi = gy_hi; v_lo = ya_lo * f1_lo; v_hi = ya_hi * f1_hi;
+                                       L.Post[rho_lo][lane] = f2_lo; L.Post[rho_hi][lane] = f2_hi; }
+                if (KIND == SCAN_GV) { q_lo = xa_lo * f2_lo; q_hi = xa_hi * f2_hi; k_lo = ya_lo * f1_lo; k_hi = ya_hi * f1_hi;
+                                       v_lo = gy_lo; v_hi = gy_hi;
+                                       pu[m_lo] = ya_lo * u_e * xa_lo; pu[m_hi] = ya_hi * u_e * xa_hi; }
+                if (QS) {
+                    const unsigned qh = pack_bf16(q_lo, q_hi);
+                    st_bf16_pair(&L.Qh[rho_lo][lane], &L.Qh[rho_hi][lane], qh);
+                    st_bf16_pair(&L.Ql[rho_lo][lane], &L.Ql[rho_hi][lane], pack_bf16(q_lo - bf16_lo(qh), q_hi - bf16_hi(qh)));
+                } else {
+                    st_bf16_pair(&L.Qh[rho_lo][lane], &L.Qh[rho_hi][lane], xbits);
                 }
-                vth[e >> 3][e & 7] = vh;
-                vtl[e >> 3][e & 7] = (__bf16)(valv - (float)vh);
+                if (KS) {
+                    const unsigned kh = pack_bf16(k_lo, k_hi);
+                    const unsigned kl = pack_bf16(k_lo - bf16_lo(kh), k_hi - bf16_hi(kh));
+                    st_bf16_pair(&L.Kh[rho_lo][lane], &L.Kh[rho_hi][lane], kh);
+                    st_bf16_pair(&L.Kl[rho_lo][lane], &L.Kl[rho_hi][lane], kl);
+                    kthw[e_lo >> 1] = kh;
+                    ktlw[e_lo >> 1] = kl;
+                } else {
+                    st_bf16_pair(&L.Kh[rho_lo][lane], &L.Kh[rho_hi][lane], xbits);
+                    kthw[e_lo >> 1] = xbits;
+                }
+                const unsigned vh = pack_bf16(v_lo, v_hi);
+                vthw[e_lo >> 1] = vh;
+                vtlw[e_lo >> 1] = pack_bf16(v_lo - bf16_lo(vh), v_hi - bf16_hi(vh));
             }
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                *reinterpret_cast<bf16x8*>(&L.KTh[lane][r0 + 8 * e]) = kth[e];
-                if (KS) *reinterpret_cast<bf16x8*>(&L.KTl[lane][r0 + 8 * e]) = ktl[e];
-                *reinterpret_cast<bf16x8*>(&L.VTh[lane][r0 + 8 * e]) = vth[e];
-                *reinterpret_cast<bf16x8*>(&L.VTl[lane][r0 + 8 * e]) = vtl[e];
+                *reinterpret_cast<u32x4*>(&L.KTh[lane][r0 + 8 * e]) = u32x4{kthw[4 * e], kthw[4 * e + 1], kthw[4 * e + 2], kthw[4 * e + 3]};
+                if (KS) *reinterpret_cast<u32x4*>(&L.KTl[lane][r0 + 8 * e]) = u32x4{ktlw[4 * e], ktlw[4 * e + 1], ktlw[4 * e + 2], ktlw[4 * e + 3]};
+                *reinterpret_cast<u32x4*>(&L.VTh[lane][r0 + 8 * e]) = u32x4{vthw[4 * e], vthw[4 * e + 1], vthw[4 * e + 2], vthw[4 * e + 3]};
+                *reinterpret_cast<u32x4*>(&L.VTl[lane][r0 + 8 * e]) = u32x4{vtlw[4 * e], vtlw[4 * e + 1], vtlw[4 * e + 2], vtlw[4 * e + 3]};
             }
             if (KIND == SCAN_GV && ASC) {                                 // bonus_n = sum_j r_n[j] u[j] k_n[j]
                 int idx;
@@ -249,25 +305,62 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh_, accA, 0, 0, 0);
             }
         }
+        // A[t][s] keeps s before t and takes the bonus at s = t (GV); GR and GK pick A[t][t] = v_t . gy_t up on the
+        // way.  All on the packed bf16 words with the lane's constant bit masks.
         const float bon = (KIND == SCAN_GV && ASC) ? (L.Bon[0][x] + L.Bon[1][x]) + (L.Bon[2][x] + L.Bon[3][x]) : 0.f;
+        const unsigned dgh = pack_bf16(bon, bon), dgl = pack_bf16(bon - bf16_lo(dgh), bon - bf16_lo(dgh));
         bf16x8 Ah[2], Al[2];
-        int dx = 4 * g - x;
-        asm volatile("" : "+v"(dx));
-        float dsel = 0.f;                                                 // A[t][t] (v_t . gy_t for GR, GK)
+        if (MASK_REGS) {
+            unsigned dh = 0u, dl = 0u;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            float a8[8];
+            for (int ks = 0; ks < 2; ++ks) {
+                float a8[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int r = 8 * ks + e;
-                const int sx = 8 * (r / 4) + (r % 4) + dx;                // s - x
-                a8[e] = sx < 0 ? accA[r] : (sx == 0 ? bon : 0.f);
-                if (KIND != SCAN_GV) dsel = sx == 0 ? accA[r] : dsel;
+                for (int e = 0; e < 8; ++e) a8[e] = accA[8 * ks + e];
+                bf16x8 h8, l8;
+                split8(a8, h8, l8);
+                u32x4 hw = __builtin_bit_cast(u32x4, h8), lw = __builtin_bit_cast(u32x4, l8);
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    const unsigned kw = keepw[4 * ks + pr], dw = diagw[4 * ks + pr];
+                    if (KIND != SCAN_GV) {
+                        dh |= hw[pr] & dw;
+                        dl |= lw[pr] & dw;
+                        hw[pr] &= kw;
+                        lw[pr] &= kw;
+                    } else if (ASC) {
+                        hw[pr] = (hw[pr] & kw) | (dgh & dw);
+                        lw[pr] = (lw[pr] & kw) | (dgl & dw);
+                    } else {
+                        hw[pr] &= kw;
+                        lw[pr] &= kw;
+                    }
+                }
+                Ah[ks] = __builtin_bit_cast(bf16x8, hw);
+                Al[ks] = __builtin_bit_cast(bf16x8, lw);
             }
-            split8(a8, Ah[ks], Al[ks]);
-        }
-        if (KIND != SCAN_GV) {
-            // exactly one lane of each column x holds the diagonal element; both waves computed the same A
+            if (KIND != SCAN_GV) {
+                // exactly one lane of each column x holds the diagonal element (head + tail of the split, one half
+                // of each word); both waves computed the same A
+                const float dsel = (bf16_lo(dh) + bf16_hi(dh)) + (bf16_lo(dl) + bf16_hi(dl));
+                if (((x >> 2) & 1) == g) L.Diag[x] = dsel;
+            }
+        } else {
+            int dx = 4 * g - x;
+            asm volatile("" : "+v"(dx));
+            float dsel = 0.f;                                             // A[t][t] (v_t . gy_t)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                float a8[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int r = 8 * ks + e;
+                    const int sx = 8 * (r / 4) + (r % 4) + dx;            // s - x
+                    a8[e] = sx < 0 ? accA[r] : 0.f;
+                    dsel = sx == 0 ? accA[r] : dsel;
+                }
+                split8(a8, Ah[ks], Al[ks]);
+            }
             if (((x >> 2) & 1) == g) L.Diag[x] = dsel;
         }
         // ---- MFMA 2: Out[t][o] = sum_s A[t][s] Val[s][o] ----

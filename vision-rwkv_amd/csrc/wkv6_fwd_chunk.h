@@ -59,14 +59,32 @@ constexpr float SAFE_DECAY = 60.f;
 __device__ __forceinline__ bf16x8 cat8(bf16x4 a, bf16x4 b) {
     return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
-// head/tail split of eight fp32 accumulator values into two packed bf16 operands
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+constexpr float LOG2_LOG2E = 0.5287663729448977f;     // log2(log2(e))
+// two fp32 values rounded to bf16 in one register (a low, b high), and the halves widened back
+__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+__device__ __forceinline__ float bf16_lo(unsigned w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+__device__ __forceinline__ void st_bf16_pair(__bf16* lo, __bf16* hi, unsigned w) {
+    *reinterpret_cast<unsigned short*>(lo) = (unsigned short)w;
+    *reinterpret_cast<unsigned short*>(hi) = (unsigned short)(w >> 16);
+}
+
+// head/tail split of eight fp32 accumulator values into two packed bf16 operands (two values per conversion)
 __device__ __forceinline__ void split8(const float (&x)[8], bf16x8& hi, bf16x8& lo) {
+    u32x4 h, l;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const __bf16 h = (__bf16)x[e];
-        hi[e] = h;
-        lo[e] = (__bf16)(x[e] - (float)h);
+    for (int p = 0; p < 4; ++p) {
+        const unsigned w = pack_bf16(x[2 * p], x[2 * p + 1]);
+        h[p] = w;
+        l[p] = pack_bf16(x[2 * p] - bf16_lo(w), x[2 * p + 1] - bf16_hi(w));
     }
+    hi = __builtin_bit_cast(bf16x8, h);
+    lo = __builtin_bit_cast(bf16x8, l);
 }
 
 // DPP move: lane reads `v` of the lane selected by CTRL (0 where there is none).
@@ -149,23 +167,28 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     auto chunk_of = [&](int ch) { return asc ? ch : nchunk - 1 - ch; };
     const int sgn = asc ? 1 : -1, n0 = asc ? 0 : LC - 1;
     auto token_of = [&](int c, int n) { return c * LC + n0 + sgn * n; };
+    // Row offsets walk the 16 tokens of this wave's block with one scalar add each; rows past T (last chunk
+    // only) are clamped to the last row and switched off where they are used.
     auto fetch_w = [&](int ch, int C) {
-        const int c = chunk_of(ch);
+        const unsigned step = (unsigned)(sgn * C * (int)sizeof(WT)), last = (unsigned)(T - 1) * C * (unsigned)sizeof(WT);
+        unsigned so = (unsigned)token_of(chunk_of(ch), 16 * q) * C * (unsigned)sizeof(WT);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const int t = token_of(c, 16 * q + m);                        // wave-uniform: a scalar row offset
-            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(WT));
+            wraw[m] = BufRaw<sizeof(WT)>::ld(rsw, lane * (unsigned)sizeof(WT), so < last ? so : last);
+            so += step;
         }
     };
     auto fetch_rkv = [&](int ch, int C) {
-        const int c = chunk_of(ch);
+        const unsigned step = (unsigned)(sgn * C * (int)sizeof(IO)), last = (unsigned)(T - 1) * C * (unsigned)sizeof(IO);
+        unsigned so = (unsigned)token_of(chunk_of(ch), 16 * q) * C * (unsigned)sizeof(IO);
+        const unsigned vo = lane * (unsigned)sizeof(IO);
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
-            const int t = token_of(c, 16 * q + m);
-            const unsigned so = (unsigned)(t < T ? t : 0) * C * (unsigned)sizeof(IO), vo = lane * (unsigned)sizeof(IO);
-            rraw[m] = BufRaw<sizeof(IO)>::ld(rsr, vo, so);
-            kraw[m] = BufRaw<sizeof(IO)>::ld(rsk, vo, so);
-            vraw[m] = BufRaw<sizeof(IO)>::ld(rsv, vo, so);
+            const unsigned sc = so < last ? so : last;
+            rraw[m] = BufRaw<sizeof(IO)>::ld(rsr, vo, sc);
+            kraw[m] = BufRaw<sizeof(IO)>::ld(rsk, vo, sc);
+            vraw[m] = BufRaw<sizeof(IO)>::ld(rsv, vo, sc);
+            so += step;
         }
     };
     auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
@@ -178,6 +201,14 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         return y_lane + (unsigned)((c * LC + y_n0) * C * 4) + (unsigned)((8 * (r / 4) + (r % 4)) * (sgn * C * 4));
     };
     fetch_w(0, C);
+    // causal masks of the in-chunk matrix, one word per pair of accumulator registers (r = 2p low half, 2p + 1 high)
+    unsigned keepw[8], diagw[8];
+#pragma unroll
+    for (int pr = 0; pr < 8; ++pr) {
+        const int s0 = 8 * ((2 * pr) / 4) + 4 * g + ((2 * pr) % 4);     // row s of register 2p; register 2p + 1 holds s0 + 1
+        keepw[pr] = (s0 < x ? 0xffffu : 0u) | (s0 + 1 < x ? 0xffff0000u : 0u);
+        diagw[pr] = (s0 == x ? 0xffffu : 0u) | (s0 + 1 == x ? 0xffff0000u : 0u);
+    }
 
     for (int ch = 0; ch < nchunk; ++ch) {
         // =============================== stage E: elementwise =================================
@@ -188,68 +219,86 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         asm volatile("" : "+s"(Cs));
         WKV6_STAMP(0);
         fetch_rkv(ch, Cs);                                                   // used after the first barrier
-        float ld[16];
-#pragma unroll
-        for (int m = 0; m < 16; ++m) {
-            const bool ok = token_of(chunk_of(ch), 16 * q + m) < T;
-            const float fw = cvtw(wraw[m]);
-            ld[m] = ok ? (W_IS_EW ? fw : -__expf(fw)) : 0.f;
-        }
+        // log decays in log2 units: ld2 = -log2(e) exp(w) = -exp2(w log2(e) + log2(log2(e)))
+        const bool full = (chunk_of(ch) + 1) * LC <= T;                  // wave-uniform: no token of the chunk is past T
         float p[16];
-        p[0] = ld[0];
+        {
+            float e[16];
 #pragma unroll
-        for (int m = 1; m < 16; ++m) p[m] = p[m - 1] + ld[m];
+            for (int m = 0; m < 16; ++m) {
+                const float fw = cvtw(wraw[m]);
+                e[m] = W_IS_EW ? -fw * LOG2E : fast_exp2(fmaf(fw, LOG2E, LOG2_LOG2E));
+            }
+            if (!full) {
+#pragma unroll
+                for (int m = 0; m < 16; ++m)
+                    if (token_of(chunk_of(ch), 16 * q + m) >= T) e[m] = 0.f;
+            }
+            p[0] = -e[0];
+#pragma unroll
+            for (int m = 1; m < 16; ++m) p[m] = p[m - 1] - e[m];
+        }
         if (q == 0) L.Tot[lane] = p[15];
         WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
         WKV6_STAMP(2);
-        const float pref = L.Tot[lane];                                  // P_15
-        const float off = q == 1 ? pref : 0.f;
+        const float pref = L.Tot[lane];                                  // P_15 (log2 units)
+        const float dq = q == 1 ? 0.f : -pref;                           // z_m = P_m - Pref = p[m] + dq
         if (q == 1) {
-            const float p31 = p[15] + off;
-            L.C2[lane] = __expf(p31);
-            L.C3[lane] = __expf(p31 - pref);
-            if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY)) != 0ull && lane == 0) sFlag = 1;
+            const float p31 = p[15] + pref;
+            L.C2[lane] = fast_exp2(p31);
+            L.C3[lane] = fast_exp2(p[15]);
+            if (__builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag = 1;
         } else {
-            L.C1[lane] = __expf(pref);
+            L.C1[lane] = fast_exp2(pref);
         }
         {
-            bf16x8 kth[2], ktl[2], vth[2], vtl[2];
-            float rr[16], kk[16], vv[16];
+            if (!full) {                                                  // k = 0 switches a token past T off everywhere
 #pragma unroll
-            for (int m = 0; m < 16; ++m) {
-                const bool ok = token_of(chunk_of(ch), 16 * q + m) < T;
-                rr[m] = ok ? cvt(rraw[m]) : 0.f;
-                kk[m] = ok ? cvt(kraw[m]) : 0.f;
-                vv[m] = ok ? cvt(vraw[m]) : 0.f;
+                for (int m = 0; m < 16; ++m)
+                    if (token_of(chunk_of(ch), 16 * q + m) >= T) kraw[m] = RawIO{};
             }
+            unsigned kthw[8], ktlw[8], vthw[8], vtlw[8];
+            float pu[16];
+            float zp = dq;                                                // Pex_m - Pref = z_(m-1)
 #pragma unroll
-            for (int m = 0; m < 16; ++m) {
+            for (int m = 0; m < 16; m += 2) {
                 const int n = 16 * q + m;
-                const float P = p[m] + off;
-                const float f1 = __expf((m ? p[m - 1] : 0.f) + off - pref);  // exp(Pex - Pref), Pex_m = P_(m-1)
-                const float f2 = __expf(pref - P);                        // exp(Pref - P)
-                const float rt = rr[m] * f1, kt = kk[m] * f2;
-                const __bf16 rh = (__bf16)rt, kh = (__bf16)kt;
-                const __bf16 rl = (__bf16)(rt - (float)rh), kl = (__bf16)(kt - (float)kh);
-                L.Rh[n][lane] = rh; L.Rl[n][lane] = rl;
-                L.Kh[n][lane] = kh; L.Kl[n][lane] = kl;
-                kth[m >> 3][m & 7] = kh; ktl[m >> 3][m & 7] = kl;
-                const __bf16 vh = (__bf16)vv[m];
-                vth[m >> 3][m & 7] = vh;
-                if (VSPLIT) vtl[m >> 3][m & 7] = (__bf16)(vv[m] - (float)vh);
+                const float z0 = p[m] + dq, z1 = p[m + 1] + dq;
+                const float f1a = fast_exp2(zp), f2a = fast_exp2(-z0);    // exp(Pex - Pref), exp(Pref - P)
+                const float f1b = fast_exp2(z0), f2b = fast_exp2(-z1);
+                zp = z1;
+                const float r0 = cvt(rraw[m]), r1 = cvt(rraw[m + 1]), k0 = cvt(kraw[m]), k1 = cvt(kraw[m + 1]);
+                const float rt0 = r0 * f1a, rt1 = r1 * f1b, kt0 = k0 * f2a, kt1 = k1 * f2b;
+                const unsigned rh = pack_bf16(rt0, rt1), kh = pack_bf16(kt0, kt1);    // token m low, m + 1 high
+                const unsigned rl = pack_bf16(rt0 - bf16_lo(rh), rt1 - bf16_hi(rh));
+                const unsigned kl = pack_bf16(kt0 - bf16_lo(kh), kt1 - bf16_hi(kh));
+                st_bf16_pair(&L.Rh[n][lane], &L.Rh[n + 1][lane], rh);
+                st_bf16_pair(&L.Rl[n][lane], &L.Rl[n + 1][lane], rl);
+                st_bf16_pair(&L.Kh[n][lane], &L.Kh[n + 1][lane], kh);
+                st_bf16_pair(&L.Kl[n][lane], &L.Kl[n + 1][lane], kl);
+                kthw[m >> 1] = kh;
+                ktlw[m >> 1] = kl;
+                if constexpr (!VSPLIT) {
+                    vthw[m >> 1] = (unsigned)vraw[m] | ((unsigned)vraw[m + 1] << 16);   // bf16 bits as loaded
+                } else {
+                    const float v0 = cvt(vraw[m]), v1 = cvt(vraw[m + 1]);
+                    const unsigned vh = pack_bf16(v0, v1);
+                    vthw[m >> 1] = vh;
+                    vtlw[m >> 1] = pack_bf16(v0 - bf16_lo(vh), v1 - bf16_hi(vh));
+                }
+                pu[m] = r0 * uj * k0;
+                pu[m + 1] = r1 * uj * k1;
             }
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                *reinterpret_cast<bf16x8*>(&L.Kth[lane][16 * q + 8 * e]) = kth[e];
-                *reinterpret_cast<bf16x8*>(&L.Ktl[lane][16 * q + 8 * e]) = ktl[e];
-                *reinterpret_cast<bf16x8*>(&L.Vt[lane][16 * q + 8 * e]) = vth[e];
-                if (VSPLIT) *reinterpret_cast<bf16x8*>(&L.Vtl[lane][16 * q + 8 * e]) = vtl[e];
+                *reinterpret_cast<u32x4*>(&L.Kth[lane][16 * q + 8 * e]) = u32x4{kthw[4 * e], kthw[4 * e + 1], kthw[4 * e + 2], kthw[4 * e + 3]};
+                *reinterpret_cast<u32x4*>(&L.Ktl[lane][16 * q + 8 * e]) = u32x4{ktlw[4 * e], ktlw[4 * e + 1], ktlw[4 * e + 2], ktlw[4 * e + 3]};
+                *reinterpret_cast<u32x4*>(&L.Vt[lane][16 * q + 8 * e]) = u32x4{vthw[4 * e], vthw[4 * e + 1], vthw[4 * e + 2], vthw[4 * e + 3]};
+                if constexpr (VSPLIT)
+                    *reinterpret_cast<u32x4*>(&L.Vtl[lane][16 * q + 8 * e]) = u32x4{vtlw[4 * e], vtlw[4 * e + 1], vtlw[4 * e + 2], vtlw[4 * e + 3]};
             }
             if (asc) {                                                    // bonus_n = sum_j r_n[j] u[j] k_n[j]
-                float pu[16];
-#pragma unroll
-                for (int m = 0; m < 16; ++m) pu[m] = rr[m] * uj * kk[m];
                 int idx;
                 const float rs = row_sums16(pu, lane, idx);
                 L.Bon[lane >> 4][16 * q + idx] = rs;                      // the four 16-channel rows are added by the reader
@@ -287,20 +336,26 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, accA, 0, 0, 0);
             accA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh_, accA, 0, 0, 0);
         }
+        // A[t][s] keeps s < t and takes the bonus at s = t: applied to the packed bf16 words with the lane's
+        // constant bit masks (the lane holds t = x, rows s = 8(r/4) + 4g + (r%4))
         const float diag = asc ? (L.Bon[0][x] + L.Bon[1][x]) + (L.Bon[2][x] + L.Bon[3][x]) : 0.f;
+        const unsigned dgh = pack_bf16(diag, diag), dgl = pack_bf16(diag - bf16_lo(dgh), diag - bf16_lo(dgh));
         bf16x8 Ah[2], Al[2];
-        int dx = 4 * g - x;                                               // compared in place: 32 hoisted lane masks
-        asm volatile("" : "+v"(dx));                                      // would not fit the scalar registers
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             float a8[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int r = 8 * ks + e;
-                const int sx = 8 * (r / 4) + (r % 4) + dx;                // s - x with s = 8(r/4) + 4g + (r%4)
-                a8[e] = sx < 0 ? accA[r] : (sx == 0 ? diag : 0.f);        // earlier tokens; the token itself through the bonus
+            for (int e = 0; e < 8; ++e) a8[e] = accA[8 * ks + e];
+            bf16x8 h8, l8;
+            split8(a8, h8, l8);
+            u32x4 hw = __builtin_bit_cast(u32x4, h8), lw = __builtin_bit_cast(u32x4, l8);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                hw[p] = (hw[p] & keepw[4 * ks + p]) | (dgh & diagw[4 * ks + p]);
+                lw[p] = (lw[p] & keepw[4 * ks + p]) | (dgl & diagw[4 * ks + p]);
             }
-            split8(a8, Ah[ks], Al[ks]);
+            Ah[ks] = __builtin_bit_cast(bf16x8, hw);
+            Al[ks] = __builtin_bit_cast(bf16x8, lw);
         }
         // ---- MFMA 2: Y[t][i] = sum_s A[t][s] V[s][i]; contraction order = accumulator order ----
         f32x16 accY = {0};
