@@ -163,7 +163,8 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     // Both passes walk the same 32-token chunks of the token axis (the ascending pass chunk 0, 1, ..., the
     // descending pass chunk nchunk-1, ..., 0), so everything that depends on the position is wave-uniform.
     // Pass index n = 0..31 inside a chunk is token 32c + n (ascending) or 32c + 31 - n (descending); tokens
-    // past T (only in the last chunk; for the descending pass they come first) are r = k = v = 0, d = 1.
+    // past T (only in the last chunk; for the descending pass they come first) read the last row and count as
+    // k = 0, d = 1 (their own y rows are dropped by the store's range check).
     auto chunk_of = [&](int ch) { return asc ? ch : nchunk - 1 - ch; };
     const int sgn = asc ? 1 : -1, n0 = asc ? 0 : LC - 1;
     auto token_of = [&](int c, int n) { return c * LC + n0 + sgn * n; };
