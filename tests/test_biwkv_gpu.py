@@ -114,6 +114,26 @@ def test_ragged_shapes(ops, B, T, C):
         assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= TOL_16
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,T,C", [(2, 225, 64), (1, 384, 128), (2, 448, 72), (1, 449, 64), (2, 576, 128),
+                                   (1, 672, 64), (3, 600, 200), (40, 300, 512)])
+def test_two_and_three_super_chunks_16bit(ops, B, T, C, dtype):
+    """16-bit sequences of 225..672 tokens take the one-launch path that keeps a whole sequence in a workgroup's
+    registers (24- or 28-token chunks, two or three super-chunks; 320 sequences walk the persistent loop).  One
+    channel tile has parameters outside the plain-sum regime and is redone by the renormalising recurrence."""
+    from oracle import clib
+    rng = np.random.default_rng(B * 1000 + T + C)
+    k = rng.standard_normal((B, T, C), dtype=np.float32)
+    v = rng.standard_normal((B, T, C), dtype=np.float32)
+    w = rng.uniform(-5, 3, C).astype(np.float32) / T
+    u = rng.uniform(-1, 1, C).astype(np.float32) / T
+    if C > 64:
+        w[C - 3] = 2.5
+    y, kr, vr = run(ops, w, u, k, v, dtype)
+    assert np.isfinite(y).all()
+    assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= TOL_16
+
+
 def test_very_long_sequence_many_super_chunks(ops):
     """T = 9100 is 41 super-chunks: more than the carry step's on-chip table holds, so it walks the workspace
     directly; a second channel tile has parameters outside the plain-sum regime (its entries must stay untouched)."""

@@ -710,6 +710,12 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     for (tile = blockIdx.x; tile < g.n_tiles; tile += gridDim.x) t.run_robust(tile);
 }
 
+}  // namespace biwkv_fwd_detail
+}  // namespace vrwkv
+#include "biwkv_fwd_resident.h"
+namespace vrwkv {
+namespace biwkv_fwd_detail {
+
 // ------------------------------- host-side dispatch ---------------------------------
 struct Plan {
     int L = 0, S = 0, nSC = 0, VEC = 0, grid = 0;
@@ -790,6 +796,21 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
         if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
             if (!p.multi()) {
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+            } else if (sizeof(IO) == 2 && L == 28 && p.nSC <= 3 && !env_int("VRWKV_BIWKV_NO_RESIDENT")) {
+                // two or three super-chunks of 16-bit rows fit a workgroup's registers: one launch, k and v read once
+                if constexpr (sizeof(IO) == 2 && L == 28) {
+                    const int n_seq = B * p.geom.n_ctile;
+                    const int eg = env_int("VRWKV_BIWKV_GRID");
+                    const int g1 = eg > 0 ? eg : num_cus();
+                    const dim3 rgrid(g1 < n_seq ? g1 : n_seq);
+                    const bool short_chunks = T <= p.nSC * 8 * 24;        // 24-token chunks need no spills with three super-chunks
+                    const int RL = short_chunks ? 24 : 28;
+                    const dim3 rblock(((T + p.nSC * RL - 1) / (p.nSC * RL)) * WAVE);
+#define VRWKV_RESIDENT(NSC_, L_) hipLaunchKernelGGL((biwkv_fwd_resident_kernel<IO, NSC_, L_>), rgrid, rblock, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom.n_ctile, n_seq)
+                    if (p.nSC == 2) { if (short_chunks) VRWKV_RESIDENT(2, 24); else VRWKV_RESIDENT(2, 28); }
+                    else            { if (short_chunks) VRWKV_RESIDENT(3, 24); else VRWKV_RESIDENT(3, 28); }
+#undef VRWKV_RESIDENT
+                }
             } else {
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
