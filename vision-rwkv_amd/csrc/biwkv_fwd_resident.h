@@ -25,11 +25,60 @@ namespace biwkv_fwd_detail {
 // LDS accesses of the kernel below go through these helpers: their __restrict__ parameters give the accesses alias
 // scopes, and only then does the compiler leave the waits for the rows still on their way (LDS-direct loads) to the
 // hand-written s_waitcnt instead of draining every one of them before each LDS access.
-template <typename IO>
-__device__ __forceinline__ unsigned lds_row_pair(const IO* __restrict__ rows, int k_idx, int v_idx) {
-    const unsigned kb = __builtin_bit_cast(unsigned short, rows[k_idx]);
-    const unsigned vb = __builtin_bit_cast(unsigned short, rows[v_idx]);
-    return kb | (vb << 16);
+// k and v of eight (four) tokens from a wave's row region: the LDS reads are issued back to back and waited for inside
+// the same statement (the compiler does not know that the registers are still being written); k goes to the low,
+// v to the high half of one register per token.  Written with plain loads the compiler, short of registers, reads
+// token after token and waits for each.  (Loads that write one half of a register and keep the other do not exist
+// on this target: with SRAM ECC a 16-bit load clears the other half.)  Rows are 128 bytes apart.
+__device__ __forceinline__ void lds_row_octet(unsigned k_addr, unsigned v_addr, unsigned* bits) {
+    unsigned k0, k1, k2, k3, k4, k5, k6, k7, v0, v1, v2, v3, v4, v5, v6, v7;
+    asm volatile("ds_read_u16 %0, %16\n\t"
+                 "ds_read_u16 %1, %16 offset:128\n\t"
+                 "ds_read_u16 %2, %16 offset:256\n\t"
+                 "ds_read_u16 %3, %16 offset:384\n\t"
+                 "ds_read_u16 %4, %16 offset:512\n\t"
+                 "ds_read_u16 %5, %16 offset:640\n\t"
+                 "ds_read_u16 %6, %16 offset:768\n\t"
+                 "ds_read_u16 %7, %16 offset:896\n\t"
+                 "ds_read_u16 %8, %17\n\t"
+                 "ds_read_u16 %9, %17 offset:128\n\t"
+                 "ds_read_u16 %10, %17 offset:256\n\t"
+                 "ds_read_u16 %11, %17 offset:384\n\t"
+                 "ds_read_u16 %12, %17 offset:512\n\t"
+                 "ds_read_u16 %13, %17 offset:640\n\t"
+                 "ds_read_u16 %14, %17 offset:768\n\t"
+                 "ds_read_u16 %15, %17 offset:896\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(k0), "=&v"(k1), "=&v"(k2), "=&v"(k3), "=&v"(k4), "=&v"(k5), "=&v"(k6), "=&v"(k7),
+                   "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+                 : "v"(k_addr), "v"(v_addr)
+                 : "memory");
+    bits[0] = k0 | (v0 << 16); bits[1] = k1 | (v1 << 16); bits[2] = k2 | (v2 << 16); bits[3] = k3 | (v3 << 16);
+    bits[4] = k4 | (v4 << 16); bits[5] = k5 | (v5 << 16); bits[6] = k6 | (v6 << 16); bits[7] = k7 | (v7 << 16);
+}
+__device__ __forceinline__ void lds_row_quad(unsigned k_addr, unsigned v_addr, unsigned* bits) {
+    unsigned k0, k1, k2, k3, v0, v1, v2, v3;
+    asm volatile("ds_read_u16 %0, %8\n\t"
+                 "ds_read_u16 %1, %8 offset:128\n\t"
+                 "ds_read_u16 %2, %8 offset:256\n\t"
+                 "ds_read_u16 %3, %8 offset:384\n\t"
+                 "ds_read_u16 %4, %9\n\t"
+                 "ds_read_u16 %5, %9 offset:128\n\t"
+                 "ds_read_u16 %6, %9 offset:256\n\t"
+                 "ds_read_u16 %7, %9 offset:384\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(k0), "=&v"(k1), "=&v"(k2), "=&v"(k3), "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+                 : "v"(k_addr), "v"(v_addr)
+                 : "memory");
+    bits[0] = k0 | (v0 << 16); bits[1] = k1 | (v1 << 16); bits[2] = k2 | (v2 << 16); bits[3] = k3 | (v3 << 16);
+}
+// all L tokens of a wave's chunk: k rows at lds_addr, v rows LR rows further on
+template <int L, int LR>
+__device__ __forceinline__ void lds_read_rows(unsigned lds_addr, unsigned (&bits)[L]) {
+    static_assert(L % 4 == 0, "rows are read eight or four tokens at a time");
+#pragma unroll
+    for (int j = 0; j + 8 <= L; j += 8) lds_row_octet(lds_addr + j * 128, lds_addr + (LR + j) * 128, &bits[j]);
+    if constexpr (L % 8 != 0) lds_row_quad(lds_addr + (L - 4) * 128, lds_addr + (LR + L - 4) * 128, &bits[L - 4]);
 }
 template <typename IO>
 __device__ __forceinline__ void lds_put(IO* __restrict__ rows, int idx, IO val) { rows[idx] = val; }
@@ -88,7 +137,7 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
                                const IO* __restrict__ k_, const IO* __restrict__ v_, IO* __restrict__ y_,
                                float* __restrict__ ws, int T, int C, int n_ctile, int n_seq)
 {
-    static_assert(sizeof(IO) == 2, "packed register rows need 16-bit elements");
+    static_assert(sizeof(IO) == 2 && WAVE * sizeof(IO) == 128, "packed register rows need 16-bit elements (128-byte LDS rows)");
     constexpr int SMAX = 8;
     constexpr int EPL = 8, LPR = 8, RPI = 8, NI = (L + RPI - 1) / RPI, LR = NI * RPI;   // 16-byte pieces: 8 lanes per row, 8 rows per instruction
     // Row regions per wave (160 KB of LDS hold three of 24 rows or two of 32).  They are separate arrays: the compiler
@@ -183,7 +232,8 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
             // (folded into the array's address they exceed the 16-bit offset field and become 2 L registers)
             unsigned row_base = (unsigned)(wave * (2 * LR * WAVE) + lane);
             asm volatile("" : "+v"(row_base));
-            const IO* rows = region(reg) + row_base;
+            typedef __attribute__((address_space(3))) const IO* lds_cptr;
+            const unsigned rows_addr = (unsigned)(size_t)(lds_cptr)(region(reg) + row_base);     // LDS byte address of the lane's first row
             const int tw = (sc * S + wave) * L;
             // This super-chunk's rows have landed.  Loads complete in order, so the younger super-chunk on its way
             // (three regions) may stay in flight -- unless stores are pending too (first super-chunk of a sequence:
@@ -193,18 +243,13 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
             float X0[L], X1[L];
             unsigned rw_bits[L];                                          // k | v << 16, as loaded
             if (tw + L <= T) {                                            // wave-uniform: every token of the chunk exists
-#pragma unroll
-                for (int j = 0; j < L; ++j) {
-                    rw_bits[j] = lds_row_pair<IO>(rows, j * WAVE, (LR + j) * WAVE);
-                }
+                lds_read_rows<L, LR>(rows_addr, rw_bits);
             } else {
                 int nvalid = T - tw;                                      // rows past T were not written: LDS holds stale bits
                 asm volatile("" : "+v"(nvalid));                          // compared per lane: 28 scalar masks would spill
+                lds_read_rows<L, LR>(rows_addr, rw_bits);
 #pragma unroll
-                for (int j = 0; j < L; ++j) {
-                    const unsigned both = lds_row_pair<IO>(rows, j * WAVE, (LR + j) * WAVE);
-                    rw_bits[j] = j < nvalid ? both : (unsigned)ninf_bits;
-                }
+                for (int j = 0; j < L; ++j) rw_bits[j] = j < nvalid ? rw_bits[j] : (unsigned)ninf_bits;
             }
 #pragma unroll
             for (int j = 0; j < L; ++j) {
