@@ -141,12 +141,13 @@ def backward_section(torch, ops, steps, warmup):
 
 def sweep_section(torch, ops, steps, warmup):
     """Dense-prediction caller shapes (adapter backbones run groups of blocks at T = H/16 * W/16 with batch 2):
-    Bi-WKV forward and backward, fp32 I/O, per (T, C)."""
+    Bi-WKV forward and backward, fp32 I/O (forward also bf16), per (T, C); plus the VRWKV-L classification shape
+    (batch 32, 384x384 -> T=576, C=1024)."""
     dev = torch.device("cuda:0")
     rows = []
-    for Tn in (1024, 4150, 4200):
-        for Cn in (192, 384, 768, 1024):
-            Bn = 2
+    shapes = [(2, Tn, Cn) for Tn in (1024, 4150, 4200) for Cn in (192, 384, 768, 1024)] + [(32, 576, 1024)]
+    for Bn, Tn, Cn in shapes:
+        if True:
             g = torch.Generator(device="cpu").manual_seed(Tn + Cn)
             k, v, gy = (torch.randn(Bn, Tn, Cn, generator=g).to(dev) for _ in range(3))
             c = torch.arange(Cn, dtype=torch.float32)
@@ -167,8 +168,11 @@ def sweep_section(torch, ops, steps, warmup):
 
             us_f = timed(lambda: ops.bi_wkv_forward(w, u, k, v))
             us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
+            kh, vh = k.bfloat16(), v.bfloat16()
+            us_h = timed(lambda: ops.bi_wkv_forward(w, u, kh, vh))
             el = Bn * Tn * Cn * 4
             rows.append({"B": Bn, "T": Tn, "C": Cn, "fwd_us": round(us_f, 1), "fwd_GBps": round(3 * el / us_f / 1e3, 1),
+                         "fwd_bf16_us": round(us_h, 1), "fwd_bf16_GBps": round(3 * el / 2 / us_h / 1e3, 1),
                          "bwd_us": round(us_b, 1), "bwd_GBps": round(5 * el / us_b / 1e3, 1)})
     return rows
 
