@@ -91,7 +91,8 @@ class VRWKV_SpatialMix_V6(nn.Module):
         gate = self.gate(xg)
         w = self.time_decay + torch.tanh(xw @ self.time_decay_w1) @ self.time_decay_w2
         y = RUN_CUDA_RWKV6(B, T, C, self.n_head, r.contiguous(), k.contiguous(), v.contiguous(),
-                           w.float().contiguous(), self.time_faaaa.float())          # vrwkv6.py:217
+                           w.contiguous(), self.time_faaaa.float())                  # vrwkv6.py:217 (w as it is: the
+        # kernel widens a 16-bit decay logit itself, the same values the reference's `w.float()` holds)
         if self.key_norm is not None:
             y = self.key_norm(y.to(gate.dtype))
         # ln_x over each head's channels, times silu(gate) (vrwkv6.py:199, 205-211): one pass at inference
