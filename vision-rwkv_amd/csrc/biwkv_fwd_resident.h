@@ -1,10 +1,10 @@
 // Bi-WKV forward, one launch for sequences of two or three super-chunks with 16-bit I/O (included by
 // biwkv_fwd_impl.h).
 //
-// A workgroup owns a whole (batch, 64 channels) sequence of NSC super-chunks of S waves x L tokens (L = 24 keeps
-// everything in registers for three super-chunks, L = 28 reaches longer sequences at the price of a few spills).  k and v are
-// read from HBM once: every wave keeps the rows of its NSC chunks packed in registers (k in the low, v in the high
-// half of a register) between
+// A workgroup owns a whole (batch, 64 channels) sequence of NSC super-chunks of S waves x L tokens (L = 24 where the
+// sequence allows it, L = 28 for longer ones at the price of more spills with three super-chunks).  k and v are read
+// from HBM once: every wave keeps the rows of its NSC chunks packed in registers (k in the low, v in the high half
+// of a register) between
 //   phase A  per super-chunk: the wave's aggregates, one LDS exchange, and from it the carries inside the
 //            super-chunk and the super-chunk totals (every wave forms all totals, so the carries across
 //            super-chunks need no further exchange), and
@@ -22,9 +22,6 @@
 namespace vrwkv {
 namespace biwkv_fwd_detail {
 
-// LDS accesses of the kernel below go through these helpers: their __restrict__ parameters give the accesses alias
-// scopes, and only then does the compiler leave the waits for the rows still on their way (LDS-direct loads) to the
-// hand-written s_waitcnt instead of draining every one of them before each LDS access.
 // k and v of eight (four) tokens from a wave's row region: the LDS reads are issued back to back and waited for inside
 // the same statement (the compiler does not know that the registers are still being written); k goes to the low,
 // v to the high half of one register per token.  Written with plain loads the compiler, short of registers, reads
@@ -80,6 +77,7 @@ __device__ __forceinline__ void lds_read_rows(unsigned lds_addr, unsigned (&bits
     for (int j = 0; j + 8 <= L; j += 8) lds_row_octet(lds_addr + j * 128, lds_addr + (LR + j) * 128, &bits[j]);
     if constexpr (L % 8 != 0) lds_row_quad(lds_addr + (L - 4) * 128, lds_addr + (LR + L - 4) * 128, &bits[L - 4]);
 }
+// y staging and the exchange buffer (plain LDS accesses)
 template <typename IO>
 __device__ __forceinline__ void lds_put(IO* __restrict__ rows, int idx, IO val) { rows[idx] = val; }
 template <typename IO>
