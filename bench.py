@@ -367,6 +367,34 @@ def main():
             "algorithmic_bytes_per_launch": bytes_alg,
         },
     }
+    if args.io == "fp32":
+        # the same loop with bf16 tensors (secondary figure; the headline stays the fp32 one)
+        kh, vh = [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        yh = [torch.empty_like(k) for k in kh]
+        calls_h = [(w.data_ptr(), u.data_ptr(), kh[i].data_ptr(), vh[i].data_ptr(), yh[i].data_ptr(),
+                    B, T, C, _lib.VRWKV_BF16, None, 0, stream.cuda_stream) for i in range(LAYERS)]
+
+        def step_h():
+            for a in calls_h:
+                rc = fwd(*a)
+                if rc:
+                    _lib.check(rc)
+
+        for _ in range(args.warmup):
+            step_h()
+        torch.cuda.synchronize()
+        h0, h1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        h0.record(stream)
+        for _ in range(args.steps):
+            step_h()
+        h1.record(stream)
+        torch.cuda.synchronize()
+        us_h = h0.elapsed_time(h1) * 1e3 / n_launch
+        bytes_h = 3 * B * T * C * 2 + 2 * C * 4
+        out["bf16_io"] = {"us_per_call": round(us_h, 3), "GBps": round(bytes_h / us_h / 1e3, 1),
+                          "pct_hbm_peak": round(100.0 * bytes_h / us_h / 1e3 / HBM_PEAK_GBS, 2),
+                          "algorithmic_bytes_per_launch": bytes_h}
+        del kh, vh, yh
     if not args.no_cpu_baseline:
         cb, y_cpu = cpu_baseline(torch, args.cpu_calls)
         out["cpu_baseline"] = cb
