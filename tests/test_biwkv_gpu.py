@@ -134,6 +134,21 @@ def test_two_and_three_super_chunks_16bit(ops, B, T, C, dtype):
     assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= TOL_16
 
 
+def test_one_launch_and_two_kernel_paths_agree(ops, monkeypatch):
+    """The same 16-bit sequence through the one-launch kernel and through the aggregate + emit kernels: both round
+    the same fp32 arithmetic to bf16, so they may differ by an output ulp here and there, no more."""
+    B, T, C = 4, 576, 256
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((B, T, C), dtype=np.float32)
+    v = rng.standard_normal((B, T, C), dtype=np.float32)
+    w, u = baseline_wu(C, T)
+    y1, _, _ = run(ops, w, u, k, v, torch.bfloat16)
+    monkeypatch.setenv("VRWKV_BIWKV_NO_RESIDENT", "1")
+    y2, _, _ = run(ops, w, u, k, v, torch.bfloat16)
+    assert np.abs(y1 - y2).max() <= 2.0 ** -7 * np.abs(y2).max()
+    assert (y1 != y2).mean() < 0.02
+
+
 def test_very_long_sequence_many_super_chunks(ops):
     """T = 9100 is 41 super-chunks: more than the carry step's on-chip table holds, so it walks the workspace
     directly; a second channel tile has parameters outside the plain-sum regime (its entries must stay untouched)."""
