@@ -102,6 +102,42 @@ def test_chunked_scans_bf16_against_closed_form(ops, B, T, H, w_mean):
         assert rel_err(got, want) <= tol, name
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("B,T,H,w_mean", [(2, 17, 2, -0.5), (1, 33, 1, -0.5), (2, 196, 1, -0.5), (1, 100, 2, -3.0), (2, 70, 2, 0.8)])
+def test_chunked_scans_fp32_fp16_against_closed_form(ops, B, T, H, w_mean, dtype):
+    """fp32 and fp16 r, k, v take the matrix-core scans as well (split into bf16 head + tail like the computed
+    operands); reference: float64 autograd through the closed form on the inputs as the kernel sees them."""
+    from oracle import wkv6
+    rng = np.random.default_rng(T * 13 + H)
+    C = H * 64
+    r, k, v = (torch.from_numpy(rng.standard_normal((B, T, C)).astype(np.float32)).to(dtype).float().numpy() for _ in range(3))
+    gy = rng.standard_normal((B, T, C)).astype(np.float32)
+    w = rng.normal(w_mean, 0.5, (B, T, C)).astype(np.float32)
+    u = rng.normal(0, 0.1, (H, 64)).astype(np.float32)
+    (gr, gk, gv, gw, gu), *_ = run(ops, r, k, v, w, u, gy, H, dtype)
+    ref = wkv6.wkv6_grads_closed(r, k, v, w, u, H, gy)
+    for got, want, name in zip((gr, gk, gv, gw, gu), ref, ("gr", "gk", "gv", "gw", "gu")):
+        assert np.isfinite(got).all(), name
+        # gw is ld times a running difference of two sums that nearly cancel: its worst element sits a little higher
+        assert rel_err(got, want) <= (2e-3 if name == "gw" else TOL), name
+
+
+def test_sequential_sweeps_fp32(ops, monkeypatch):
+    """The sequential kernels (the fallback of flagged sequences) on their own, fp32 inputs."""
+    from oracle import wkv6
+    monkeypatch.setenv("VRWKV_WKV6_BWD_PATH", "scalar")
+    B, T, H = 2, 50, 2
+    rng = np.random.default_rng(77)
+    C = H * 64
+    r, k, v, gy = (rng.standard_normal((B, T, C)).astype(np.float32) for _ in range(4))
+    w = rng.normal(-0.5, 0.5, (B, T, C)).astype(np.float32)
+    u = rng.normal(0, 0.1, (H, 64)).astype(np.float32)
+    (gr, gk, gv, gw, gu), *_ = run(ops, r, k, v, w, u, gy, H)
+    ref = wkv6.wkv6_grads_closed(r, k, v, w, u, H, gy)
+    for got, want, name in zip((gr, gk, gv, gw, gu), ref, ("gr", "gk", "gv", "gw", "gu")):
+        assert rel_err(got, want) <= TOL, name
+
+
 def test_chunked_scans_equal_sequential_sweeps_full_size(ops, monkeypatch):
     B, T, H = 64, 196, 12
     C = H * 64

@@ -252,13 +252,13 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
     float* a = ws;                                       // (B,T,C)
     float* gu_part = ws + (size_t)B * T * C;             // (B,C)
     const dim3 grid(B * H), block(256);
-    if constexpr (std::is_same<IO, __hip_bfloat16>::value) {
+    {
         const char* path = getenv("VRWKV_WKV6_BWD_PATH");            // "scalar" forces the sequential sweeps (testing)
         if (!(path && path[0] == 's') && (long long)T * C < (1LL << 29)) {
             using namespace wkv6_detail;
             unsigned char* todo = reinterpret_cast<unsigned char*>(gu_part + (size_t)B * C);
             const dim3 blk(128);
-#define VRWKV_SCAN(KIND, DIR, OUT) hipLaunchKernelGGL((wkv6_bwd_scan_kernel<WT, KIND, DIR, EW>), grid, blk, 0, st, \
+#define VRWKV_SCAN(KIND, DIR, OUT) hipLaunchKernelGGL((wkv6_bwd_scan_kernel<IO, WT, KIND, DIR, EW>), grid, blk, 0, st, \
                                                       rr, kk, vv, ww, u, gy, OUT, a, gw, gu_part, todo, T, C, H)
             VRWKV_SCAN(SCAN_GR, 1, gr); VRWKV_SCAN(SCAN_GK, 1, gk); VRWKV_SCAN(SCAN_GV, 1, gv);
             VRWKV_SCAN(SCAN_GR, 0, gr); VRWKV_SCAN(SCAN_GK, 0, gk); VRWKV_SCAN(SCAN_GV, 0, gv);

@@ -1,4 +1,4 @@
-// wkv6 backward, chunked matrix-core scans for gfx950 (bf16 MFMA, fp32 accumulate; bf16 r, k, v).
+// wkv6 backward, chunked matrix-core scans for gfx950 (bf16 MFMA, fp32 accumulate; r, k, v in bf16, fp16 or fp32).
 //
 // One causal pass of the forward (tokens in pass order n, state S_n before token n, d_n = exp(ld_n)):
 //   y_n = r_n (diag(u) k_n v_n^T + S_n),   S_{n+1} = diag(d_n) S_n + k_n v_n^T
@@ -21,7 +21,8 @@
 //   GV: Q = kt, Kc = rt, Val = gy, state read * c3[j] (rows), update c2[j], c1[j] (rows);  gv = Out
 // GR and GK contract over the value channel i and own output columns j (the state is kept transposed, so its
 // decay is a per-lane factor); GV contracts over j like the forward.  The state never leaves the accumulator
-// registers; computed operands are split into bf16 head + tail (hh + ht + th), loaded bf16 ones are exact.
+// registers; computed operands (and fp16 / fp32 inputs) are split into bf16 head + tail (hh + ht + th), loaded
+// bf16 ones are exact.
 //
 // One 128-thread workgroup per (b,h) and pass; the descending pass is launched first and writes, the
 // ascending pass adds (old values fetched behind the matrix stage).  A sequence with a chunk that decays by
@@ -45,10 +46,10 @@ struct __attribute__((aligned(16))) ScanLds {
 };
 
 // DIR 0: ascending pass (bonus u, adds to the outputs).  DIR 1: descending pass (writes them).
-template <typename WT, int KIND, int DIR, bool W_IS_EW>
+template <typename IO, typename WT, int KIND, int DIR, bool W_IS_EW>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfloat16* __restrict__ k_,
-                          const __hip_bfloat16* __restrict__ v_, const WT* __restrict__ w_,
+void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
+                          const IO* __restrict__ v_, const WT* __restrict__ w_,
                           const float* __restrict__ u_, const float* __restrict__ gy_,
                           float* __restrict__ out_,        // gr / gk / gv
                           float* __restrict__ a_,          // GR: written; GK: read
@@ -56,11 +57,12 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                           float* __restrict__ gu_part,     // GR, DIR 0
                           unsigned char* __restrict__ todo, int T, int C, int H)
 {
-    using IO = __hip_bfloat16;
+    constexpr bool EXACT = __is_same(IO, __hip_bfloat16);  // r, k, v are bf16 values as loaded (fp16 / fp32 inputs are split in two)
+    constexpr unsigned ES = (unsigned)sizeof(IO);
     constexpr bool REV = KIND != SCAN_GR;                  // scan order = reverse pass order
     constexpr bool TT = KIND != SCAN_GV;                   // transposed state: contraction over i, output columns j
-    constexpr bool QS = KIND != SCAN_GK;                   // Q is computed (gy, kt) -> split; v is exact
-    constexpr bool KS = KIND != SCAN_GR;                   // Kc is computed (gy, rt) -> split; v is exact
+    constexpr bool QS = KIND != SCAN_GK || !EXACT;         // Q is computed (gy, kt) -> split; bf16 v is exact
+    constexpr bool KS = KIND != SCAN_GR || !EXACT;         // Kc is computed (gy, rt) -> split; bf16 v is exact
     constexpr bool ASC = DIR == 0;
     constexpr bool LL = KIND != SCAN_GV;                   // tail x tail products too: gw is a difference of these sums
     __shared__ ScanLds<QS, KS> L;
@@ -81,9 +83,9 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
     if (threadIdx.x == 0) sFlag = 0;
     __syncthreads();
 
-    using RawIO = typename BufRaw<2>::type;
+    using RawIO = typename BufRaw<sizeof(IO)>::type;
     using RawW = typename BufRaw<sizeof(WT)>::type;
-    const unsigned span_io = (unsigned)(((size_t)(T - 1) * C + HN) * 2);
+    const unsigned span_io = (unsigned)(((size_t)(T - 1) * C + HN) * ES);
     const unsigned span_w = (unsigned)(((size_t)(T - 1) * C + HN) * sizeof(WT));
     const unsigned span_f = (unsigned)(((size_t)(T - 1) * C + HN) * 4);
     const __amdgpu_buffer_rsrc_t rsr = make_rsrc(r_ + base, span_io), rsk = make_rsrc(k_ + base, span_io),
@@ -91,7 +93,7 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                                  rsg = make_rsrc(gy_ + base, span_f), rso = make_rsrc(out_ + base, span_f);
     const __amdgpu_buffer_rsrc_t rsa = make_rsrc((KIND != SCAN_GV ? a_ : out_) + base, span_f);
     const __amdgpu_buffer_rsrc_t rsgw = make_rsrc((KIND == SCAN_GK ? gw_ : out_) + base, span_f);
-    auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, 2); return to_f32(t); };
+    auto cvt = [](RawIO raw) { IO t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
     auto cvtw = [](RawW raw) { WT t; __builtin_memcpy(&t, &raw, sizeof(t)); return to_f32(t); };
 
     // Chunks are 32-token blocks of the token axis.  The scan walks them upwards when (ascending pass) !=
@@ -153,10 +155,10 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
 #pragma unroll
             for (int m = 0; m < 16; ++m) {
                 const unsigned sc = so < last ? so : last;
-                const unsigned vo = lane * 2u;
-                if (KIND == SCAN_GR) { xraw[m] = BufRaw<2>::ld(rsv, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsk, vo, sc * 2u); }
-                if (KIND == SCAN_GK) { xraw[m] = BufRaw<2>::ld(rsv, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsr, vo, sc * 2u); }
-                if (KIND == SCAN_GV) { xraw[m] = BufRaw<2>::ld(rsk, vo, sc * 2u); yraw[m] = BufRaw<2>::ld(rsr, vo, sc * 2u); }
+                const unsigned vo = lane * ES;
+                if (KIND == SCAN_GR) { xraw[m] = BufRaw<ES>::ld(rsv, vo, sc * ES); yraw[m] = BufRaw<ES>::ld(rsk, vo, sc * ES); }
+                if (KIND == SCAN_GK) { xraw[m] = BufRaw<ES>::ld(rsv, vo, sc * ES); yraw[m] = BufRaw<ES>::ld(rsr, vo, sc * ES); }
+                if (KIND == SCAN_GV) { xraw[m] = BufRaw<ES>::ld(rsk, vo, sc * ES); yraw[m] = BufRaw<ES>::ld(rsr, vo, sc * ES); }
                 graw[m] = BufRaw<4>::ld(rsg, lane * 4u, sc * 4u);
                 so += step;
             }
@@ -221,12 +223,13 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
                 const float xa_lo = cvt(xraw[m_lo]), xa_hi = cvt(xraw[m_hi]);
                 const float ya_lo = cvt(yraw[m_lo]), ya_hi = cvt(yraw[m_hi]);
                 const float gy_lo = __builtin_bit_cast(float, graw[m_lo]), gy_hi = __builtin_bit_cast(float, graw[m_hi]);
-                const unsigned xbits = (unsigned)xraw[m_lo] | ((unsigned)xraw[m_hi] << 16);   // bf16 pair as loaded
+                unsigned xbits = 0u;                                      // bf16 pair as loaded
+                if constexpr (EXACT) xbits = (unsigned)xraw[m_lo] | ((unsigned)xraw[m_hi] << 16);
                 // per scan: Q, Kc, Val of this (token, channel); exact bf16 inputs keep their bits
                 float q_lo, q_hi, k_lo, k_hi, v_lo, v_hi;
-                if (KIND == SCAN_GR) { q_lo = gy_lo; q_hi = gy_hi; v_lo = ya_lo * f2_lo; v_hi = ya_hi * f2_hi;
+                if (KIND == SCAN_GR) { q_lo = gy_lo; q_hi = gy_hi; k_lo = xa_lo; k_hi = xa_hi; v_lo = ya_lo * f2_lo; v_hi = ya_hi * f2_hi;
                                        L.Post[rho_lo][lane] = f1_lo; L.Post[rho_hi][lane] = f1_hi; }
-                if (KIND == SCAN_GK) { k_lo = gy_lo; k_hi = gy_hi; v_lo = ya_lo * f1_lo; v_hi = ya_hi * f1_hi;
+                if (KIND == SCAN_GK) { q_lo = xa_lo; q_hi = xa_hi; k_lo = gy_lo; k_hi = gy_hi; v_lo = ya_lo * f1_lo; v_hi = ya_hi * f1_hi;
                                        L.Post[rho_lo][lane] = f2_lo; L.Post[rho_hi][lane] = f2_hi; }
                 if (KIND == SCAN_GV) { q_lo = xa_lo * f2_lo; q_hi = xa_hi * f2_hi; k_lo = ya_lo * f1_lo; k_hi = ya_hi * f1_hi;
                                        v_lo = gy_lo; v_hi = gy_hi;
@@ -285,8 +288,8 @@ void wkv6_bwd_scan_kernel(const __hip_bfloat16* __restrict__ r_, const __hip_bfl
         for (int r = 0; r < 16; ++r) {
             if (KIND != SCAN_GK) prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
             if (KIND != SCAN_GV) {
-                rraw[r] = BufRaw<2>::ld(rsr, row_off(cc, r, Cs, 2), 0);
-                kraw[r] = BufRaw<2>::ld(rsk, row_off(cc, r, Cs, 2), 0);
+                rraw[r] = BufRaw<ES>::ld(rsr, row_off(cc, r, Cs, ES), 0);
+                kraw[r] = BufRaw<ES>::ld(rsk, row_off(cc, r, Cs, ES), 0);
             }
         }
         // ---- MFMA 1: A^T: acc[s][t] = sum_c Kc[s][c] Q[t][c]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
