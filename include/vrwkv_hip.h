@@ -145,7 +145,7 @@ int vrwkv_rowfuse_bwd(const void* a, const void* other, const void* ln_weight, c
  *   maa: (5, C) fp32 (time_maa_w, _k, _v, _r, _g).
  * vrwkv_groupnorm_gate: jit_func_2 (:205-211), out = GroupNorm(y) * silu(gate) with groups of `group` consecutive
  *   channels per row (ln_x = GroupNorm(n_head, C) on the (B*T, C) view); y: (rows, C) fp32 (as the operator returns
- *   it) or io_dtype; gate, out: (rows, C), gn_weight, gn_bias: (C,) of io_dtype (bf16 or fp16).
+ *   it) or io_dtype; gate, out: (rows, C), gn_weight, gn_bias: (C,) of io_dtype (fp32, bf16 or fp16; fp32 only beside an fp32 y).
  * All tensors 16-byte aligned, C a multiple of 8 (4 for fp32 maa_mix).  The reference has no native code here. */
 int vrwkv_maa_mix(const void* x, const void* sx, const void* m, const float* maa, void* const* out,
                   long long rows, int C, int io_dtype, void* hip_stream);

@@ -259,9 +259,9 @@ def test_vrwkv6_mix_kernels_against_tensor_ops(B, T, C, dtype):
     ref = ops.ops.maa_mix_tensor_ops(x.float(), sx.float(), m.float(), [a.float() for a in maas])
     for g, r in zip(got, ref):
         assert g.dtype == dtype and (g.float() - r).abs().max().item() <= tol * r.abs().max().item()
-    if dtype != torch.float32:
+    if C % 64 == 0:
         H = C // 64
-        for ydt in (torch.float32, dtype):
+        for ydt in {torch.float32, dtype}:
             y = (3 * torch.randn(B, T, C, device=dev) + 1).to(ydt)
             gate = torch.randn(B, T, C, device=dev).to(dtype)
             w, b = torch.randn(C, device=dev).to(dtype), torch.randn(C, device=dev).to(dtype)
@@ -391,9 +391,9 @@ def test_vrwkv6_mix_backward_against_autograd(B, T, C, dtype):
         assert a.grad.shape == a.shape
         check("gmaa", a.grad, a2.grad)
 
-    if dtype != torch.float32:
+    if C % 64 == 0:
         H = C // 64
-        for ydt in (torch.float32, dtype):
+        for ydt in {torch.float32, dtype}:
             y = (3 * torch.randn(B, T, C, device=dev) + 1).to(ydt).requires_grad_(True)
             gate = torch.randn(B, T, C, device=dev).to(dtype).requires_grad_(True)
             w = (1 + 0.3 * torch.randn(C, device=dev)).to(dtype).requires_grad_(True)

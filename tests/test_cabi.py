@@ -93,7 +93,7 @@ def test_elementwise_entry_points_validate_without_device(lib):
     gp[1] = None
     assert qb(one, one, gp, 3, one, one, 2, 196, 768, 14, 14, 1, 192, 0, 1, one, need, None) == 1   # a null gradient
     gg = lib.vrwkv_groupnorm_gate
-    assert gg(one, one, one, one, one, 4, 128, 64, 1e-5, 0, 0, None) == 2                      # fp32 gate / output
+    assert gg(one, one, one, one, one, 4, 128, 64, 1e-5, 1, 0, None) == 2                      # fp32 gate beside a bf16 y
     assert gg(one, one, one, one, one, 4, 128, 48, 1e-5, 0, 1, None) == 3                      # C not a multiple of the group
     assert gg(one, one, one, one, one, 4, 96, 24, 1e-5, 0, 1, None) == 3                       # group not 8..128 in powers of two
     assert b"group" in lib.vrwkv_last_error()
@@ -109,7 +109,7 @@ def test_elementwise_entry_points_validate_without_device(lib):
     gb = lib.vrwkv_groupnorm_gate_bwd
     assert lib.vrwkv_groupnorm_gate_bwd_workspace_bytes(100, 768) == 4 * 2 * 768 * 4          # one partial row pair per 32 rows
     assert gb(one, one, one, one, one, one, one, None, 4, 128, 64, 1e-5, 0, 1, None, 0, None) == 1    # gparam is null
-    assert gb(one, one, one, one, one, one, one, one, 4, 128, 64, 1e-5, 0, 0, None, 0, None) == 2     # fp32 gate
+    assert gb(one, one, one, one, one, one, one, one, 4, 128, 64, 1e-5, 2, 0, None, 0, None) == 2     # fp32 gate beside an fp16 y
     assert gb(one, one, one, one, one, one, one, one, 4, 2048, 64, 1e-5, 0, 1, None, 0, None) == 3    # more than 1024 channels
     assert gb(one, one, one, one, one, one, one, one, 4, 128, 64, 1e-5, 0, 1, None, 0, None) == 5     # workspace missing
 

@@ -51,6 +51,26 @@ void maa_mix_kernel(const IO* __restrict__ x_, const IO* __restrict__ sx_, const
     }
 }
 
+// Eight consecutive elements widened to fp32: one 16-byte vector of a 16-bit type, two of fp32.
+template <typename T>
+__device__ __forceinline__ void load8(const T* __restrict__ p, float (&out)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        load_vec<T, 4>(p, *reinterpret_cast<float(*)[4]>(&out[0]));
+        load_vec<T, 4>(p + 4, *reinterpret_cast<float(*)[4]>(&out[4]));
+    } else {
+        load_vec<T, 8>(p, out);
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* __restrict__ p, const float (&in)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        store_vec<T, 4>(p, *reinterpret_cast<const float(*)[4]>(&in[0]));
+        store_vec<T, 4>(p + 4, *reinterpret_cast<const float(*)[4]>(&in[4]));
+    } else {
+        store_vec<T, 8>(p, in);
+    }
+}
+
 // One wave per token; a lane owns 8 consecutive channels per step, so a group of 64 channels is 8 neighbouring lanes.
 template <typename YT, typename IO, int GL>                   // GL = lanes per group = group / 8
 __global__ __launch_bounds__(256)
@@ -66,12 +86,7 @@ void groupnorm_gate_kernel(const YT* __restrict__ y_, const IO* __restrict__ g_,
         const bool ok = p < nchunk;                           // whole groups: the lanes of a group agree
         const size_t e0 = (size_t)row * C + (size_t)(ok ? p : 0) * 8;
         float y[8];
-        if constexpr (sizeof(YT) == 4) {
-            load_vec<YT, 4>(y_ + e0, *reinterpret_cast<float(*)[4]>(&y[0]));
-            load_vec<YT, 4>(y_ + e0 + 4, *reinterpret_cast<float(*)[4]>(&y[4]));
-        } else {
-            load_vec<YT, 8>(y_ + e0, y);
-        }
+        load8<YT>(y_ + e0, y);
         float s = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) s += y[e];
@@ -87,15 +102,15 @@ void groupnorm_gate_kernel(const YT* __restrict__ y_, const IO* __restrict__ g_,
         if (!ok) continue;
         const int c = p * 8;
         float g[8], w[8], b[8], r[8];
-        load_vec<IO, 8>(g_ + e0, g);
-        load_vec<IO, 8>(w_ + c, w);
-        load_vec<IO, 8>(b_ + c, b);
+        load8<IO>(g_ + e0, g);
+        load8<IO>(w_ + c, w);
+        load8<IO>(b_ + c, b);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float gate = g[e] * fast_rcp(1.f + fast_exp2(-g[e] * LOG2E));      // silu
             r[e] = fmaf((y[e] - mean) * rstd, w[e], b[e]) * gate;
         }
-        store_vec<IO, 8>(out_ + e0, r);
+        store8<IO>(out_ + e0, r);
     }
 }
 
@@ -206,7 +221,7 @@ void groupnorm_gate_bwd_kernel(const YT* __restrict__ y_, const IO* __restrict__
         const int p = st * WAVE + lane;
 #pragma unroll
         for (int e = 0; e < 8; ++e) { w[st][e] = 0.f; b[st][e] = 0.f; acc_w[st][e] = 0.f; acc_b[st][e] = 0.f; }
-        if (p < nchunk) { load_vec<IO, 8>(w_ + p * 8, w[st]); load_vec<IO, 8>(b_ + p * 8, b[st]); }
+        if (p < nchunk) { load8<IO>(w_ + p * 8, w[st]); load8<IO>(b_ + p * 8, b[st]); }
     }
     const long long row0 = ((long long)blockIdx.x * (blockDim.x >> 6) + wave) * GN_RPW;
     for (int rr = 0; rr < GN_RPW; ++rr) {
@@ -219,14 +234,9 @@ void groupnorm_gate_bwd_kernel(const YT* __restrict__ y_, const IO* __restrict__
             const bool ok = p < nchunk;                       // whole groups: the lanes of a group agree
             const size_t e0 = (size_t)row * C + (size_t)(ok ? p : 0) * 8;
             float y[8], gt[8], g[8];
-            if constexpr (sizeof(YT) == 4) {
-                load_vec<YT, 4>(y_ + e0, *reinterpret_cast<float(*)[4]>(&y[0]));
-                load_vec<YT, 4>(y_ + e0 + 4, *reinterpret_cast<float(*)[4]>(&y[4]));
-            } else {
-                load_vec<YT, 8>(y_ + e0, y);
-            }
-            load_vec<IO, 8>(gate_ + e0, gt);
-            load_vec<IO, 8>(g_ + e0, g);
+            load8<YT>(y_ + e0, y);
+            load8<IO>(gate_ + e0, gt);
+            load8<IO>(g_ + e0, g);
             float s = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) s += y[e];
@@ -261,13 +271,8 @@ void groupnorm_gate_bwd_kernel(const YT* __restrict__ y_, const IO* __restrict__
             float gy[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) gy[e] = rstd * (t[e] - m1 - xh[e] * m2);
-            if constexpr (sizeof(YT) == 4) {
-                store_vec<YT, 4>(gy_ + e0, *reinterpret_cast<float(*)[4]>(&gy[0]));
-                store_vec<YT, 4>(gy_ + e0 + 4, *reinterpret_cast<float(*)[4]>(&gy[4]));
-            } else {
-                store_vec<YT, 8>(gy_ + e0, gy);
-            }
-            store_vec<IO, 8>(ggate_ + e0, gg);
+            store8<YT>(gy_ + e0, gy);
+            store8<IO>(ggate_ + e0, gg);
         }
     }
     // the four waves' channel sums are added in wave order and written as this workgroup's partial rows
@@ -364,8 +369,8 @@ extern "C" int vrwkv_groupnorm_gate(const void* y, const void* gate, const void*
         set_error("groupnorm_gate: bad arguments (rows=%lld C=%d group=%d)", rows, C, group);
         return VRWKV_INVALID_ARG;
     }
-    if ((io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16) || (y_dtype != VRWKV_F32 && y_dtype != io_dtype)) {
-        set_error("groupnorm_gate: gate / out must be bf16 or fp16 and y fp32 or that same type (got %d, %d)", io_dtype, y_dtype);
+    if ((io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16 && io_dtype != VRWKV_F32) || (y_dtype != VRWKV_F32 && y_dtype != io_dtype)) {
+        set_error("groupnorm_gate: gate / out must be fp32, bf16 or fp16 and y fp32 or that same type (got %d, %d)", io_dtype, y_dtype);
         return VRWKV_UNSUPPORTED_DTYPE;
     }
     if (C % group != 0 || group % 8 != 0 || rows > 0x7fffffffLL * 4) {
@@ -377,6 +382,7 @@ extern "C" int vrwkv_groupnorm_gate(const void* y, const void* gate, const void*
         return VRWKV_INVALID_ARG;
     }
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    if (io_dtype == VRWKV_F32) return launch_gn<float, float>(y, gate, gn_weight, gn_bias, out, rows, C, group, eps, st);
     if (io_dtype == VRWKV_BF16) {
         if (y_dtype == VRWKV_F32) return launch_gn<float, __hip_bfloat16>(y, gate, gn_weight, gn_bias, out, rows, C, group, eps, st);
         return launch_gn<__hip_bfloat16, __hip_bfloat16>(y, gate, gn_weight, gn_bias, out, rows, C, group, eps, st);
@@ -450,8 +456,8 @@ extern "C" int vrwkv_groupnorm_gate_bwd(const void* y, const void* gate, const v
         set_error("groupnorm_gate_bwd: bad arguments (rows=%lld C=%d group=%d)", rows, C, group);
         return VRWKV_INVALID_ARG;
     }
-    if ((io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16) || (y_dtype != VRWKV_F32 && y_dtype != io_dtype)) {
-        set_error("groupnorm_gate_bwd: gate / gradients must be bf16 or fp16 and y fp32 or that same type (got %d, %d)", io_dtype, y_dtype);
+    if ((io_dtype != VRWKV_BF16 && io_dtype != VRWKV_F16 && io_dtype != VRWKV_F32) || (y_dtype != VRWKV_F32 && y_dtype != io_dtype)) {
+        set_error("groupnorm_gate_bwd: gate / gradients must be fp32, bf16 or fp16 and y fp32 or that same type (got %d, %d)", io_dtype, y_dtype);
         return VRWKV_UNSUPPORTED_DTYPE;
     }
     if (C % group != 0 || group % 8 != 0 || C > GN_STEPS * WAVE * 8 || rows > 0x7fffffffLL * 32) {
@@ -470,6 +476,7 @@ extern "C" int vrwkv_groupnorm_gate_bwd(const void* y, const void* gate, const v
     }
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
     float* part = static_cast<float*>(workspace);
+    if (io_dtype == VRWKV_F32) return launch_gn_bwd<float, float>(y, gate, gn_weight, gn_bias, gout, gy, ggate, gparam, part, rows, C, group, eps, st);
     if (io_dtype == VRWKV_BF16) {
         if (y_dtype == VRWKV_F32) return launch_gn_bwd<float, __hip_bfloat16>(y, gate, gn_weight, gn_bias, gout, gy, ggate, gparam, part, rows, C, group, eps, st);
         return launch_gn_bwd<__hip_bfloat16, __hip_bfloat16>(y, gate, gn_weight, gn_bias, gout, gy, ggate, gparam, part, rows, C, group, eps, st);

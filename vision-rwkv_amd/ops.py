@@ -512,12 +512,12 @@ def _groupnorm_gate_launch(y, gate, w, b, group, eps):
 def groupnorm_gate(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
     """GroupNorm(n_groups, C) of every token of y (fp32 as RUN_CUDA_RWKV6 returns it, or gate's dtype) times
     silu(gate), in one HIP kernel (vrwkv6.py:199, 205-211), and one backward kernel under autograd (C <= 1024);
-    16-bit gate / output; tensor ops otherwise."""
+    tensor ops for other shapes."""
     C = y.shape[-1]
     group = C // n_groups if n_groups > 0 and C % n_groups == 0 else 0
     tensors = [y, gate, gn_weight, gn_bias]
     need_grad = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
-    fits = (ROW_FUSE_ENABLED and y.is_cuda and gate.dtype in (torch.bfloat16, torch.float16) and y.shape == gate.shape
+    fits = (ROW_FUSE_ENABLED and y.is_cuda and gate.dtype in (torch.float32, torch.bfloat16, torch.float16) and y.shape == gate.shape
             and y.dtype in (torch.float32, gate.dtype) and group in (8, 16, 32, 64, 128) and y.numel() > 0
             and not (need_grad and C > 1024))
     if not fits:
