@@ -1,0 +1,113 @@
+"""Edge cases of the two WKV operators on the GPU: empty batches, one- and two-token sequences, and the
+closed forms those reduce to (no oracle call is needed for them: the expected values are textbook).
+
+  Bi-WKV, T = 1: the only weight is the bonus term, so y = v exactly (up to the output rounding).
+  Bi-WKV, T = 2: y_0 = (e^{u+k_0} v_0 + e^{k_1} v_1) / (e^{u+k_0} + e^{k_1})  (neighbours have decay exponent 0).
+  wkv6,  T = 1: y[i] = (sum_j r[j] u[j] k[j]) v[i] per head.
+  wkv6,  T = 2: y_0 = (r_0 . (u k_0)) v_0 + (r_0 . k_1) v_1  (adjacent tokens: empty decay product).
+Tolerances: 1e-4 fp32, 1e-2 16-bit I/O (Bi-WKV); 1e-3 (wkv6) of max(|ref|, rms(ref)).
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import vision_rwkv_amd
+    assert torch.cuda.is_available()
+    return vision_rwkv_amd
+
+
+@pytest.mark.parametrize("shape", [(0, 196, 768), (4, 0, 64)])
+def test_biwkv_empty_inputs(ops, shape):
+    C = shape[2]
+    w = torch.randn(C, device=DEV, requires_grad=True)
+    u = torch.randn(C, device=DEV, requires_grad=True)
+    k = torch.randn(*shape, device=DEV, requires_grad=True)
+    v = torch.randn(*shape, device=DEV, requires_grad=True)
+    y = ops.RUN_CUDA(w, u, k, v)
+    assert tuple(y.shape) == shape and y.dtype == torch.float32
+    y.sum().backward()
+    torch.cuda.synchronize()
+    assert k.grad.shape == k.shape and v.grad.shape == v.shape
+    assert torch.count_nonzero(w.grad).item() == 0 and torch.count_nonzero(u.grad).item() == 0
+
+
+@pytest.mark.parametrize("shape", [(0, 196, 128), (2, 0, 64)])
+def test_wkv6_empty_inputs(ops, shape):
+    B, T, C = shape
+    H = C // 64
+    r, k, v, w = (torch.randn(*shape, device=DEV, requires_grad=True) for _ in range(4))
+    u = torch.randn(H, 64, device=DEV, requires_grad=True)
+    y = ops.RUN_CUDA_RWKV6(B, T, C, H, r, k, v, w, u)
+    assert tuple(y.shape) == shape and y.dtype == torch.float32
+    y.sum().backward()
+    torch.cuda.synchronize()
+    assert r.grad.shape == r.shape and w.grad.shape == w.shape
+    assert tuple(u.grad.shape) == (H, 64) and torch.count_nonzero(u.grad).item() == 0
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 1e-2), (torch.float16, 1e-2)])
+@pytest.mark.parametrize("B,C", [(3, 192), (1, 37), (5, 768)])
+def test_biwkv_one_and_two_tokens(ops, B, C, dtype, tol):
+    g = torch.Generator(device="cpu").manual_seed(B * 1000 + C)
+    w = (torch.rand(C, generator=g) * 8 - 5).to(DEV)
+    u = torch.randn(C, generator=g).to(DEV)
+    for T in (1, 2):
+        k = torch.randn(B, T, C, generator=g).to(DEV).to(dtype)
+        v = torch.randn(B, T, C, generator=g).to(DEV).to(dtype)
+        y = ops.bi_wkv_forward(w / T, u / T, k, v).double().cpu().numpy()
+        kd, vd, ud = k.double().cpu().numpy(), v.double().cpu().numpy(), (u / T).double().cpu().numpy()
+        if T == 1:
+            ref = vd
+        else:
+            ref = np.empty_like(vd)
+            for t in (0, 1):
+                a, b = np.exp(ud + kd[:, t]), np.exp(kd[:, 1 - t])
+                ref[:, t] = (a * vd[:, t] + b * vd[:, 1 - t]) / (a + b)
+        assert rel_err(y, ref) <= tol, (T, rel_err(y, ref))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_wkv6_one_and_two_tokens(ops, dtype):
+    B, H = 3, 2
+    C = H * 64
+    g = torch.Generator(device="cpu").manual_seed(7)
+    u = (0.1 * torch.randn(H, 64, generator=g)).to(DEV)
+    for T in (1, 2):
+        r, k, v = (torch.randn(B, T, C, generator=g).to(DEV).to(dtype) for _ in range(3))
+        w = (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(DEV)
+        y = ops.RUN_CUDA_RWKV6(B, T, C, H, r, k, v, w, u).double().cpu().numpy().reshape(B, T, H, 64)
+        rd, kd, vd = (x.double().cpu().numpy().reshape(B, T, H, 64) for x in (r, k, v))
+        ud = u.double().cpu().numpy()[None]
+        ref = np.empty_like(vd)
+        for t in range(T):
+            ref[:, t] = (rd[:, t] * ud * kd[:, t]).sum(-1, keepdims=True) * vd[:, t]
+            if T == 2:
+                ref[:, t] += (rd[:, t] * kd[:, 1 - t]).sum(-1, keepdims=True) * vd[:, 1 - t]
+        assert rel_err(y, ref) <= 1e-3, (T, rel_err(y, ref))
+
+
+def test_backward_gradient_sum_identities_full_size(ops):
+    """Size-independent identities of the Bi-WKV gradients at the VRWKV-B shape: y is unchanged by k -> k + const, so
+    sum_t gk = 0, and the weights of a token's output sum to one, so sum_t gv = sum_t gy (both per (b, c))."""
+    B, T, C = 64, 196, 768
+    g = torch.Generator(device="cpu").manual_seed(11)
+    c = torch.arange(C, dtype=torch.float32)
+    w = ((-5 + 8 * c / (C - 1)) / T).to(DEV)
+    u = ((np.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T).to(DEV)
+    k = torch.randn(B, T, C, generator=g).to(DEV)
+    v = torch.randn(B, T, C, generator=g).to(DEV)
+    gy = torch.randn(B, T, C, generator=g).to(DEV)
+    gw, gu, gk, gv = ops.bi_wkv_backward(w, u, k, v, gy)
+    scale = gk.abs().sum(1).double()
+    assert (gk.double().sum(1).abs() <= 1e-4 * scale + 1e-6).all()
+    diff = (gv.double().sum(1) - gy.double().sum(1)).abs()
+    assert (diff <= 1e-4 * gy.abs().sum(1).double() + 1e-6).all()
+    assert torch.isfinite(gw).all() and torch.isfinite(gu).all()
