@@ -211,11 +211,7 @@ struct BiwkvTile {
             mu[e] = wu.u[e] * LOG2E;
             bad = bad || !(fabsf(om[e]) * (float)(T + 1) + fabsf(mu[e]) <= FAST_LIMIT);
         }
-#ifdef VRWKV_PROBE_NO_ROBUST
-        return false;
-#else
         return __builtin_amdgcn_ballot_w64(bad) != 0ull;
-#endif
     }
 
     // Fast path of one tile from the packed registers K, V; in the middle (once K, V have been

@@ -143,7 +143,6 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         int Cs = C;
         asm volatile("" : "+s"(Cs));                       // keep row offsets out of the loop-invariant scalars
         const int cc = chunk_of(ch);
-        WKV6_STAMP(0);
         // =============================== stage E: elementwise =================================
         // wave q prepares pass indices n = 16q .. 16q+15 of the chunk; lane = channel
         RawIO xraw[16], yraw[16];                          // the two bf16 tensors this scan needs here
@@ -183,9 +182,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             for (int m = 1; m < 16; ++m) p[m] = p[m - 1] - e[m];
         }
         if (q == 0) L.Tot[lane] = p[15];
-        WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
-        WKV6_STAMP(2);
         const float pref = L.Tot[lane];                                  // P_15 (log2 units)
         const float dq = q == 1 ? 0.f : -pref;                           // z_m = P_m - Pref = p[m] + dq
         if (q == 1) {
@@ -269,9 +266,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 L.Bon[lane >> 4][r0 + (REV ? 15 - idx : idx)] = rs;
             }
         }
-        WKV6_STAMP(3);
         lds_barrier();                                                   // (2)
-        WKV6_STAMP(4);
         if (sFlag) {                                                      // out of range: left to the sequential kernels
             if (threadIdx.x == 0) todo[bh] = 1;
             return;
@@ -448,7 +443,6 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + cu[e] * accM[4 * r4 + e];
             }
         }
-        WKV6_STAMP(5);
         // ================================== epilogue ==================================
         if (KIND == SCAN_GV) {
 #pragma unroll
@@ -510,9 +504,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 xcarry = before;
             }
         }
-        WKV6_STAMP(6);
         lds_barrier();                                                   // (3) LDS is rewritten by the next chunk
-        WKV6_STAMP(7);
     }
     if (KIND == SCAN_GR && ASC) {
         gu_acc += __shfl_xor(gu_acc, 32);

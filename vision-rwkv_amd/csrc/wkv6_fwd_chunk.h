@@ -38,10 +38,6 @@
 #include "wkv6_fwd_scalar.h"
 #include <type_traits>
 
-#ifndef WKV6_STAMP
-#define WKV6_STAMP(phase)                 // timing hook of the micro-benchmarks; nothing in the library build
-#endif
-
 namespace vrwkv {
 namespace wkv6_detail {
 
@@ -218,7 +214,6 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // occupy ~100 scalar registers and spill.
         int Cs = C;
         asm volatile("" : "+s"(Cs));
-        WKV6_STAMP(0);
         fetch_rkv(ch, Cs);                                                   // used after the first barrier
         // log decays in log2 units: ld2 = -log2(e) exp(w) = -exp2(w log2(e) + log2(log2(e)))
         const bool full = (chunk_of(ch) + 1) * LC <= T;                  // wave-uniform: no token of the chunk is past T
@@ -240,9 +235,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             for (int m = 1; m < 16; ++m) p[m] = p[m - 1] - e[m];
         }
         if (q == 0) L.Tot[lane] = p[15];
-        WKV6_STAMP(1);
         lds_barrier();                                                   // (1)
-        WKV6_STAMP(2);
         const float pref = L.Tot[lane];                                  // P_15 (log2 units)
         const float dq = q == 1 ? 0.f : -pref;                           // z_m = P_m - Pref = p[m] + dq
         if (q == 1) {
@@ -305,9 +298,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 L.Bon[lane >> 4][16 * q + idx] = rs;                      // the four 16-channel rows are added by the reader
             }
         }
-        WKV6_STAMP(3);
         lds_barrier();                                                   // (2)
-        WKV6_STAMP(4);
         if (sFlag) { bail = true; break; }                               // out of range: redo with the exact recurrence
 
         if (ch + 1 < nchunk) fetch_w(ch + 1, Cs);                             // next chunk's decays, behind the matrix stage
@@ -422,7 +413,6 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 for (int e = 0; e < 4; ++e) S[4 * r4 + e] = c2[e] * S[4 * r4 + e] + c3[e] * accM[4 * r4 + e];
             }
         }
-        WKV6_STAMP(5);
         // ---- y: store (sum with the other pass's value where it came first); on a tie the descending pass
         //      stores here and the ascending pass adds after the barrier ----
         if (!y_tie) {
@@ -432,12 +422,9 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         }
         // end of the step: every LDS read of this chunk is done, and the stores above become visible
         // to the other pass of this workgroup
-        WKV6_STAMP(6);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        WKV6_STAMP(7);
         __builtin_amdgcn_s_barrier();                                    // (3)
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        WKV6_STAMP(8);
         if (y_tie) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r, Cs), 0));
