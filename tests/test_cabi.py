@@ -123,3 +123,18 @@ def test_python_boundary_errors_without_device():
         ops.bi_wkv_forward(w, w, k, k)
     with pytest.raises(TypeError):
         ops.RUN_CUDA(w, w, k)
+
+
+def test_bench_refuses_more_than_one_gpu_and_has_no_cpu_path():
+    """bench.py runs on one GPU: --gpus 2 exits with a message instead of a number, and without a GPU the timed path
+    refuses to run (nothing falls back to the CPU oracle)."""
+    import subprocess
+    import sys
+    import torch
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr + r.stdout and "{" not in r.stdout
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "1"],
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode != 0 and "needs a GPU" in r.stderr and "{" not in r.stdout
