@@ -111,3 +111,51 @@ def test_backward_gradient_sum_identities_full_size(ops):
     diff = (gv.double().sum(1) - gy.double().sum(1)).abs()
     assert (diff <= 1e-4 * gy.abs().sum(1).double() + 1e-6).all()
     assert torch.isfinite(gw).all() and torch.isfinite(gu).all()
+
+
+def _offset_copy(t, n=1):
+    """Same values in storage that starts n elements into an allocation: contiguous, but not 16-byte aligned."""
+    buf = torch.empty(t.numel() + n, dtype=t.dtype, device=t.device)
+    out = buf[n:].view(t.shape)
+    out.copy_(t)
+    assert out.is_contiguous() and out.data_ptr() % 16 != 0
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,C", [(3, 196, 192), (2, 500, 128)])
+def test_biwkv_tensors_that_are_not_16_byte_aligned(ops, B, T, C, dtype):
+    """k, v, gy views that start one element into their allocation take the kernels without 16-byte row staging;
+    results agree with the aligned call (same arithmetic, other load path): 1e-5 of the tensor's scale."""
+    g = torch.Generator(device="cpu").manual_seed(T + C)
+    c = torch.arange(C, dtype=torch.float32)
+    w = ((-5 + 8 * c / (C - 1)) / T).to(DEV)
+    u = ((np.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T).to(DEV)
+    k, v, gy = (torch.randn(B, T, C, generator=g).to(DEV).to(dtype) for _ in range(3))
+    y0 = ops.bi_wkv_forward(w, u, k, v)
+    g0 = ops.bi_wkv_backward(w, u, k, v, gy)
+    ko, vo, gyo = _offset_copy(k), _offset_copy(v), _offset_copy(gy)
+    y1 = ops.bi_wkv_forward(w, u, ko, vo)
+    g1 = ops.bi_wkv_backward(w, u, ko, vo, gyo)
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -7
+    assert (y1.float() - y0.float()).abs().max() <= tol * y0.float().abs().max()
+    for a, b in zip(g1, g0):
+        assert (a.float() - b.float()).abs().max() <= max(tol, 1e-4) * b.float().abs().max()
+
+
+def test_wkv6_tensors_that_are_not_16_byte_aligned(ops):
+    B, T, H = 2, 100, 2
+    C = H * 64
+    g = torch.Generator(device="cpu").manual_seed(3)
+    r, k, v = (torch.randn(B, T, C, generator=g).to(DEV).to(torch.bfloat16) for _ in range(3))
+    w = (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(DEV)
+    gy = torch.randn(B, T, C, generator=g).to(DEV)
+    u = (0.1 * torch.randn(H, 64, generator=g)).to(DEV)
+    y0 = ops.wkv6_forward(B, T, C, H, r, k, v, w, u)
+    g0 = ops.wkv6_backward(B, T, C, H, r, k, v, w, u, gy)
+    ro, ko, vo, wo, gyo = (_offset_copy(t) for t in (r, k, v, w, gy))
+    y1 = ops.wkv6_forward(B, T, C, H, ro, ko, vo, wo, u)
+    g1 = ops.wkv6_backward(B, T, C, H, ro, ko, vo, wo, u, gyo)
+    assert torch.equal(y1, y0)
+    for a, b in zip(g1, g0):
+        assert torch.equal(a, b)
