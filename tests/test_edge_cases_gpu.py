@@ -159,3 +159,52 @@ def test_wkv6_tensors_that_are_not_16_byte_aligned(ops):
     assert torch.equal(y1, y0)
     for a, b in zip(g1, g0):
         assert torch.equal(a, b)
+
+
+def test_tensors_larger_than_4_gib(ops):
+    """Maximum sizes: B*T*C*4 bytes beyond 2^32 (7200 x 196 x 768), all four operators.  No oracle run at this size:
+    the kernels are deterministic and treat every (b, channel tile) / (b, head) alone, so the last and the first
+    batch elements of the big call must equal, bit for bit, a call on those elements alone (which the other tests
+    pin to the oracle); a 32-bit offset anywhere would break exactly that.  Plus sum_t gk = 0 and finiteness overall."""
+    if torch.cuda.get_device_properties(0).total_memory < 100e9:
+        pytest.skip("needs about 50 GB of device memory")
+    B, T, C = 7200, 196, 768
+    H = C // 64
+    assert B * T * C * 4 > 2 ** 32
+    c = torch.arange(C, dtype=torch.float32)
+    w = ((-5 + 8 * c / (C - 1)) / T).to(DEV)
+    u = ((np.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T).to(DEV)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    k, v, gy = (torch.randn(B, T, C, device=DEV, generator=g) for _ in range(3))
+    tail, head = slice(B - 3, B), slice(0, 3)
+    part = lambda t, s: t[s].contiguous()
+
+    y = ops.bi_wkv_forward(w, u, k, v)
+    for s in (tail, head):
+        assert torch.equal(y[s], ops.bi_wkv_forward(w, u, part(k, s), part(v, s)))
+    assert torch.isfinite(y).all()
+    del y
+    gw, gu, gk, gv = ops.bi_wkv_backward(w, u, k, v, gy)
+    _, _, gk2, gv2 = ops.bi_wkv_backward(w, u, part(k, tail), part(v, tail), part(gy, tail))
+    assert torch.equal(gk[tail], gk2) and torch.equal(gv[tail], gv2)
+    assert gk.double().sum(1).abs().max().item() <= 1e-3
+    assert torch.isfinite(gw).all() and torch.isfinite(gu).all()
+    del gk, gv, gk2, gv2
+    torch.cuda.empty_cache()
+
+    r = torch.randn(B, T, C, device=DEV, generator=g).bfloat16()
+    kb, vb = k.bfloat16(), v.bfloat16()
+    del k, v
+    wl = torch.randn(B, T, C, device=DEV, generator=g) * 0.5 - 0.5
+    u6 = 0.1 * torch.randn(H, 64, device=DEV, generator=g)
+    y = ops.wkv6_forward(B, T, C, H, r, kb, vb, wl, u6)
+    assert torch.equal(y[tail], ops.wkv6_forward(3, T, C, H, part(r, tail), part(kb, tail), part(vb, tail), part(wl, tail), u6))
+    assert torch.isfinite(y).all()
+    del y
+    big = ops.wkv6_backward(B, T, C, H, r, kb, vb, wl, u6, gy)
+    small = ops.wkv6_backward(3, T, C, H, part(r, tail), part(kb, tail), part(vb, tail), part(wl, tail), u6, part(gy, tail))
+    for a, b in zip(big[:4], small[:4]):
+        assert torch.equal(a[tail], b)
+    assert torch.isfinite(big[4]).all()
+    del big, small, r, kb, vb, wl, gy
+    torch.cuda.empty_cache()
