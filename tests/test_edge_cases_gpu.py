@@ -208,3 +208,38 @@ def test_tensors_larger_than_4_gib(ops):
     assert torch.isfinite(big[4]).all()
     del big, small, r, kb, vb, wl, gy
     torch.cuda.empty_cache()
+
+
+def test_elementwise_kernels_beyond_4_gib(ops):
+    """The fused shift + mix, row epilogue, GroupNorm x gate and five-mix kernels on 7200 x 196 x 768 fp32 tensors
+    (4.3 GB each): every output row depends on its own batch element only, so the last batch elements must equal,
+    bit for bit, a call on those elements alone (pinned against tensor ops by the other tests)."""
+    if torch.cuda.get_device_properties(0).total_memory < 100e9:
+        pytest.skip("needs about 55 GB of device memory")
+    O = ops.ops
+    B, T, C = 7200, 196, 768
+    g = torch.Generator(device=DEV).manual_seed(2)
+    tail = slice(B - 2, B)
+    part = lambda t: t[tail].contiguous()
+    x, other = (torch.randn(B, T, C, device=DEV, generator=g) for _ in range(2))
+    lw, lb = (torch.randn(C, device=DEV, generator=g) for _ in range(2))
+    mixes = [torch.rand(C, device=DEV, generator=g) for _ in range(3)]
+    with torch.no_grad():
+        outs = ops.q_shift_mix(x, mixes, patch_resolution=(14, 14))
+        for a, b in zip(outs, ops.q_shift_mix(part(x), mixes, patch_resolution=(14, 14))):
+            assert torch.equal(a[tail], b)
+        del outs
+        r = ops.row_fuse(x, other, lw, lb, post=O.POST_SIGMOID_GATE)
+        assert torch.equal(r[tail], ops.row_fuse(part(x), part(other), lw, lb, post=O.POST_SIGMOID_GATE))
+        assert torch.isfinite(r).all()
+        r = ops.groupnorm_gate(x, other, lw, lb, 12)
+        assert torch.equal(r[tail], ops.groupnorm_gate(part(x), part(other), lw, lb, 12))
+        assert torch.isfinite(r).all()
+        del r
+        m = torch.randn(5, B, T, C, device=DEV, generator=g)
+        maas = [torch.rand(C, device=DEV, generator=g) for _ in range(5)]
+        outs = ops.maa_mix(x, other, m, maas)
+        for a, b in zip(outs, ops.maa_mix(part(x), part(other), m[:, tail].contiguous(), maas)):
+            assert torch.equal(a[tail], b)
+    del outs, m, x, other
+    torch.cuda.empty_cache()
