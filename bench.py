@@ -89,6 +89,12 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
         "mfma_issued_tflops": round(mfma_flops / (us * 1e-6) / 1e12, 2),
         "pct_bf16_mfma_peak_end_to_end": round(100.0 * mfma_flops / (us * 1e-6) / 2.5e15, 3),
     }
+    # end to end the operator's arithmetic intensity (issued MFMA flop per mandatory byte) is below the machine
+    # balance, so min(MFMA peak, AI x HBM peak) is the HBM leg: report the fraction of it as well
+    io_bytes = Bw * Tw * Cw * (3 * r.element_size() + w.element_size() + 4) + u.numel() * 4
+    out["roofline"] = {"bound": "hbm", "achieved": round(io_bytes / (us * 1e-6) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                       "frac": round(io_bytes / (us * 1e-6) / 8e12, 4), "algorithmic_bytes_per_launch": io_bytes,
+                       "flop_per_byte_issued": round(mfma_flops / io_bytes, 1)}
     if with_cpu:
         from oracle import torch_eager
         bs = 4
