@@ -72,12 +72,15 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
         ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(steps):
-        y = ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
-    e1.record()
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / steps
+    reps = []
+    for _ in range(5):                                             # median of five timed loops of `steps` calls
+        e0.record()
+        for _ in range(steps):
+            y = ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
+        e1.record()
+        torch.cuda.synchronize()
+        reps.append(e0.elapsed_time(e1) * 1e3 / steps)
+    us = sorted(reps)[len(reps) // 2]
     nchunk = (Tw + 31) // 32
     # per chunk, pass and value half (one wave): 36 MFMA 32x32x16 = 36 * 32768 flop
     mfma_flops = Bw * Hw * 2 * nchunk * 2 * 36 * 32768
