@@ -133,9 +133,11 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(stage + L * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
         }
     };
-    if (STAGED && (int)blockIdx.x < n_tiles) issue_stage(blockIdx.x);
+    // workgroups are dealt round-robin to the 8 XCDs: per round, XCD x takes a contiguous eighth of the tiles
+    const int wg = (gridDim.x & 7) == 0 ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+    if (STAGED && wg < n_tiles) issue_stage(wg);
 
-    for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    for (int tile = wg; tile < n_tiles; tile += gridDim.x) {
         const int ctile = tile % n_ctile;
         const int sc = (tile / n_ctile) % nSC, b = tile / n_ctile / nSC;
         const int c0 = ctile * WAVE + lane;

@@ -159,12 +159,14 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
     typedef __attribute__((address_space(3))) void* lds_ptr;
     auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
 
-    // Super-chunk number m of this workgroup's stream (sequence blockIdx.x + (m / NSC) gridDim.x, super-chunk m % NSC):
+    // workgroups are dealt round-robin to the 8 XCDs: per round, XCD x takes a contiguous eighth of the sequences
+    const int wg = (gridDim.x & 7) == 0 ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+    // Super-chunk number m of this workgroup's stream (sequence wg + (m / NSC) gridDim.x, super-chunk m % NSC):
     // its rows for this wave -> region m % NREG.  Nothing is issued past the last sequence.
-    auto stream_exists = [&](int m) { return blockIdx.x + (m / NSC) * gridDim.x < (unsigned)n_seq; };
+    auto stream_exists = [&](int m) { return wg + (m / NSC) * (int)gridDim.x < n_seq; };
     auto issue_rows = [&](int m, int reg) {
         if (!stream_exists(m)) return;
-        const int seq = blockIdx.x + (m / NSC) * gridDim.x, sc = m % NSC;
+        const int seq = wg + (m / NSC) * (int)gridDim.x, sc = m % NSC;
         const int ctile = seq % n_ctile, b = seq / n_ctile;
         const size_t slab = (size_t)b * T * C;
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_ + slab, bytes), rv = make_rsrc(v_ + slab, bytes);
@@ -188,7 +190,7 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
     __syncthreads();
 
     int n = 0;                                   // stream position
-    int seq = blockIdx.x;
+    int seq = wg;
     if (seq >= n_seq) return;
 #pragma unroll
     for (int m = 0; m < NREG - 1; ++m) issue_rows(m, m % NREG);
