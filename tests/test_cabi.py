@@ -138,3 +138,20 @@ def test_bench_refuses_more_than_one_gpu_and_has_no_cpu_path():
         r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "1"],
                            capture_output=True, text=True, timeout=300)
         assert r.returncode != 0 and "needs a GPU" in r.stderr and "{" not in r.stdout
+
+
+def test_extension_module_stand_ins_and_torch_ops_namespaces():
+    """The reference's three extension modules (bi_wkv.cpp:49-57, wkv_op.cpp:13-21, wkv6_op.cpp:13-21) have stand-ins
+    with the same function names, also reachable through torch.ops."""
+    import torch
+    import vision_rwkv_amd as ops
+    assert set(ops.ext.REGISTERED) == {"bi_wkv", "wkv", "wkv6"}
+    for mod, names in ((ops.ext.bi_wkv, ("bi_wkv_forward", "bi_wkv_backward")), (ops.ext.wkv, ("forward", "backward")),
+                       (ops.ext.wkv6, ("forward", "backward"))):
+        for n in names:
+            assert callable(getattr(mod, n))
+    assert torch.ops.bi_wkv.bi_wkv_forward is not None and torch.ops.wkv.forward is not None
+    assert torch.ops.wkv6.backward is not None
+    k = torch.randn(2, 8, 64)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ops.ext.wkv.forward(2, 8, 64, torch.zeros(64), torch.zeros(64), k, k, torch.empty_like(k))

@@ -25,13 +25,23 @@ def _check_input(x, name):
         raise RuntimeError(f"{name} must be contiguous")
 
 
+def _check_out(t, name, shape, dtype, like):
+    """A caller-allocated result (the legacy / wkv6 extension interfaces pass them in)."""
+    if not (t.is_cuda and t.is_contiguous() and t.device == like.device):
+        raise RuntimeError(f"{name} must be a contiguous CUDA tensor on the inputs' device")
+    if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
+        raise RuntimeError(f"{name} must have shape {tuple(shape)} and dtype {dtype}")
+    return t
+
+
 def _stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def bi_wkv_forward(w, u, k, v):
+def bi_wkv_forward(w, u, k, v, out=None):
     """Extension-level entry (bi_wkv.cpp:23-33): w,u (C,) fp32; k,v (B,T,C) of one dtype
-    (fp32, bf16 or fp16); returns y (B,T,C) of that dtype.  State and arithmetic are fp32."""
+    (fp32, bf16 or fp16); returns y (B,T,C) of that dtype.  State and arithmetic are fp32.
+    out: a caller-allocated y (the legacy interface, wkv_op.cpp:6-8)."""
     for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v")):
         _check_input(t, n)
     if k.dim() != 3 or v.shape != k.shape:
@@ -45,7 +55,7 @@ def bi_wkv_forward(w, u, k, v):
         raise RuntimeError("k and v must share one of float32 / bfloat16 / float16")
     L = _lib.lib()
     dt = _DT[k.dtype]
-    y = torch.empty_like(k)
+    y = torch.empty_like(k) if out is None else _check_out(out, "y", k.shape, k.dtype, k)
     if y.numel() == 0:
         return y
     ws_bytes = L.vrwkv_biwkv_fwd_workspace_bytes(B, T, C, dt)
@@ -57,10 +67,10 @@ def bi_wkv_forward(w, u, k, v):
     return y
 
 
-def bi_wkv_backward(w, u, k, v, gy):
+def bi_wkv_backward(w, u, k, v, gy, out=None):
     """Extension-level entry (bi_wkv.cpp:35-47): w,u (C,) fp32; k,v,gy (B,T,C) of one dtype;
     returns [gw, gu, gk, gv] with gw, gu (C,) fp32 summed over batch and tokens and gk, gv of the
-    dtype of k."""
+    dtype of k.  out: caller-allocated (gw, gu, gk, gv)."""
     for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v"), (gy, "gy")):
         _check_input(t, n)
     if k.dim() != 3 or v.shape != k.shape or gy.shape != k.shape:
@@ -72,10 +82,14 @@ def bi_wkv_backward(w, u, k, v, gy):
         raise RuntimeError("k, v and gy must share one of float32 / bfloat16 / float16")
     L = _lib.lib()
     dt = _DT[k.dtype]
-    gw = torch.empty(C, dtype=torch.float32, device=k.device)
-    gu = torch.empty(C, dtype=torch.float32, device=k.device)
-    gk = torch.empty_like(k)
-    gv = torch.empty_like(k)
+    if out is None:
+        gw = torch.empty(C, dtype=torch.float32, device=k.device)
+        gu = torch.empty(C, dtype=torch.float32, device=k.device)
+        gk = torch.empty_like(k)
+        gv = torch.empty_like(k)
+    else:
+        gw, gu = (_check_out(t, n, (C,), torch.float32, k) for t, n in zip(out[:2], ("gw", "gu")))
+        gk, gv = (_check_out(t, n, k.shape, k.dtype, k) for t, n in zip(out[2:], ("gk", "gv")))
     if k.numel() == 0:
         return [gw.zero_(), gu.zero_(), gk, gv]
     ws_bytes = L.vrwkv_biwkv_bwd_workspace_bytes(B, T, C, dt)
@@ -149,7 +163,7 @@ def RUN_CUDA(*args):
 HEAD_SIZE = 64   # vrwkv6.py:23
 
 
-def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False):
+def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False, out=None):
     """Extension-level entry (wkv6_op.cpp:7-9): r,k,v (B,T,C) fp32/bf16/fp16, w (B,T,C) fp32 or
     that dtype, u (H,64); returns y (B,T,C) fp32.  With w_is_ew=False, w is the raw decay logit
     (the kernel applies d = exp(-exp(w))); with True it is ew = -exp(w_raw) as the reference
@@ -166,7 +180,8 @@ def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False):
         raise RuntimeError("w must be float32 or have the dtype of r, k, v")
     uf = u if u.dtype == torch.float32 else u.float()
     L = _lib.lib()
-    y = torch.empty((B, T, C), device=r.device, dtype=torch.float32)
+    y = (torch.empty((B, T, C), device=r.device, dtype=torch.float32) if out is None
+         else _check_out(out, "y", (B, T, C), torch.float32, r))      # the reference passes y in (wkv6_op.cpp:7-9)
     if y.numel() == 0:
         return y
     ws_bytes = L.vrwkv_wkv6_fwd_workspace_bytes(B, T, C, H)
@@ -179,7 +194,7 @@ def wkv6_forward(B, T, C, H, r, k, v, w, u, w_is_ew=False):
     return y
 
 
-def wkv6_backward(B, T, C, H, r, k, v, w, u, gy, w_is_ew=False):
+def wkv6_backward(B, T, C, H, r, k, v, w, u, gy, w_is_ew=False, out=None):
     """Extension-level entry (wkv6_op.cpp:10-12): returns (gr, gk, gv, gw) as (B,T,C) fp32 and gu as
     (H,64) fp32 (already summed over the batch); gw is the gradient w.r.t. the raw decay logit."""
     for t, n in ((r, "r"), (k, "k"), (v, "v"), (w, "w"), (u, "u"), (gy, "gy")):
@@ -193,9 +208,13 @@ def wkv6_backward(B, T, C, H, r, k, v, w, u, gy, w_is_ew=False):
     uf = u if u.dtype == torch.float32 else u.float()
     gyf = gy if gy.dtype == torch.float32 else gy.float()
     L = _lib.lib()
-    mk = lambda: torch.empty((B, T, C), device=r.device, dtype=torch.float32)
-    gr, gk, gv, gw = mk(), mk(), mk(), mk()
-    gu = torch.empty((H, C // H), device=r.device, dtype=torch.float32)
+    if out is None:
+        mk = lambda: torch.empty((B, T, C), device=r.device, dtype=torch.float32)
+        gr, gk, gv, gw = mk(), mk(), mk(), mk()
+        gu = torch.empty((H, C // H), device=r.device, dtype=torch.float32)
+    else:                                                             # caller-allocated (gr, gk, gv, gw, gu)
+        gr, gk, gv, gw = (_check_out(t, n, (B, T, C), torch.float32, r) for t, n in zip(out[:4], ("gr", "gk", "gv", "gw")))
+        gu = _check_out(out[4], "gu", (H, C // H), torch.float32, r)
     if gr.numel() == 0:
         return gr, gk, gv, gw, gu.zero_()
     ws_bytes = L.vrwkv_wkv6_bwd_workspace_bytes(B, T, C, H)
