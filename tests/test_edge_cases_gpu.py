@@ -243,3 +243,45 @@ def test_elementwise_kernels_beyond_4_gib(ops):
             assert torch.equal(a[tail], b)
     del outs, m, x, other
     torch.cuda.empty_cache()
+
+
+def test_concurrent_calls_from_threads_on_their_own_streams(ops):
+    """The library keeps no state between calls besides a thread-local error string, and every call brings its own
+    workspace: four host threads, each on its own stream, repeat the long-sequence Bi-WKV forward (which uses a
+    workspace) and the wkv6 forward, and must reproduce the single-threaded results bit for bit."""
+    import threading
+    B, T, C, H = 2, 700, 128, 2
+    g = torch.Generator(device="cpu").manual_seed(9)
+    c = torch.arange(C, dtype=torch.float32)
+    w = ((-5 + 8 * c / (C - 1)) / T).to(DEV)
+    u = ((np.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T).to(DEV)
+    sets = []
+    for _ in range(4):
+        k, v, r = (torch.randn(B, T, C, generator=g).to(DEV) for _ in range(3))
+        wl = (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(DEV)
+        sets.append((k, v, r, wl))
+    u6 = (0.1 * torch.randn(H, 64, generator=g)).to(DEV)
+    ref = [(ops.bi_wkv_forward(w, u, k, v), ops.wkv6_forward(B, T, C, H, r, k, v, wl, u6)) for k, v, r, wl in sets]
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(i):
+        try:
+            k, v, r, wl = sets[i]
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for _ in range(10):
+                    y = ops.bi_wkv_forward(w, u, k, v)
+                    y6 = ops.wkv6_forward(B, T, C, H, r, k, v, wl, u6)
+                st.synchronize()
+            if not (torch.equal(y, ref[i][0]) and torch.equal(y6, ref[i][1])):
+                errors.append(f"thread {i}: results differ")
+        except Exception as e:                                        # noqa: BLE001 - reported below
+            errors.append(f"thread {i}: {e!r}")
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=60)
+    assert not errors, errors
