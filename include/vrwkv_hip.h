@@ -36,6 +36,13 @@ enum { VRWKV_F32 = 0, VRWKV_BF16 = 1, VRWKV_F16 = 2 };
 int vrwkv_version(void);                 /* major*10000 + minor*100 + patch */
 const char* vrwkv_last_error(void);      /* thread-local, never NULL */
 
+/* Tuning / testing switches, process-wide (no counterpart in the reference).  Names: "biwkv_l", "biwkv_s",
+ * "biwkv_grid", "biwkv_no_stage", "biwkv_no_resident", "biwkv_bwd_serial", "wkv6_fwd_scalar", "wkv6_bwd_scalar",
+ * "wkv6_bwd_unfused"; 0 = default behaviour.  The initial value of <name> is that of the environment variable
+ * VRWKV_<NAME> when the library first looks at any switch; the entry points never read the environment afterwards. */
+int vrwkv_set_option(const char* name, int value);
+int vrwkv_get_option(const char* name, int* value);
+
 /* ---- Bi-WKV forward -------------------------------------------------------------------
  * Replaces bi_wkv_forward(w,u,k,v) -> y
  *   (classification/mmcls_custom/models/backbones/cuda_new/bi_wkv.cpp:23-33,

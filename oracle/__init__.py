@@ -13,6 +13,8 @@ biwkv.py       Bi-WKV forward in float64: O(T^2) closed form, two-pass
 wkv6.py        bidirectional RWKV-6 scan in float64: sequential recurrence,
                O(T^2) cumulative-log-decay closed form, autograd gradients.
 qshift.py      q_shift / q_shift_multihead as explicit index loops.
+blocks.py      the element-wise block steps around the operators (row epilogues,
+               VRWKV6 token mixes, GroupNorm x gate), row by row in float64.
 torch_eager.py the same recurrences as PyTorch CPU-eager fp32 loops over T
                (what the benchmark times as its CPU baseline).
 c/             plain-C restatement of the recurrences (double accumulators),
@@ -24,8 +26,13 @@ Pinning status (what each function is checked against, see tests/test_oracle_*):
       convexity, k-shift invariance, reversal symmetry, channel independence.
   wkv6_scan / wkv6_closed   : mutual agreement, d==1 linear-attention einsum,
       d==0 three-token form, T=1, head independence, reversal symmetry.
-  q_shift loops             : zero-border / pass-through invariants and a
-      tensor-slicing restatement.
+  q_shift loops             : zero-border / pass-through invariants, a
+      tensor-slicing restatement with channel-group bounds stated by hand
+      (equal quarters and the unequal groups of C % 4 != 0).
+  blocks                    : hand-computed rows, torch LayerNorm / GroupNorm
+      in float64, step-order checks.
+  C backward routines       : autograd through the closed forms, finite
+      differences and the sum identities (tests/test_oracle_c.py).
 The reference ships no golden vectors or tests for these operators, so the
 fixtures under tests/golden/ are produced from the float64 closed forms here.
 """

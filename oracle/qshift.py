@@ -23,15 +23,17 @@ def _source(direction, y, x, Hp, Wp, s):
 
 
 def q_shift_loops(x, shift_pixel, gamma, patch_resolution):
-    """x: (B,T,C) -> (B,T,C); channel quarter q of width int(C*gamma) moves in direction q."""
+    """x: (B,T,C) -> (B,T,C); channel group q = [int(C*gamma*q), int(C*gamma*(q+1))) moves in direction q."""
     x = np.asarray(x)
     B, T, C = x.shape
     Hp, Wp = patch_resolution
     assert Hp * Wp == T and gamma <= 0.25
-    g = int(C * gamma)
+    # the reference cuts the channel axis at int(C*gamma), int(C*gamma*2), int(C*gamma*3), int(C*gamma*4)
+    # (vrwkv.py:72-76); for C*gamma not an integer the groups are not four equal quarters
+    bounds = [int(C * gamma), int(C * gamma * 2), int(C * gamma * 3), int(C * gamma * 4)]
     out = np.zeros_like(x)
     for c in range(C):
-        direction = c // g if (g > 0 and c < 4 * g) else 4
+        direction = next((d for d, hi in enumerate(bounds) if c < hi), 4)
         for yy in range(Hp):
             for xx in range(Wp):
                 src = _source(direction, yy, xx, Hp, Wp, shift_pixel)

@@ -35,3 +35,18 @@ def rel_err(y, ref, floor_frac=1.0):
     ref = np.asarray(ref, np.float64)
     floor = floor_frac * np.sqrt(np.mean(ref * ref)) + 1e-300
     return float(np.max(np.abs(y - ref) / np.maximum(np.abs(ref), floor)))
+
+
+@pytest.fixture
+def force():
+    """force(name, value): sets a tuning / testing switch of the library (vrwkv_set_option) until the test ends."""
+    import vision_rwkv_amd as ops
+    saved = {}
+
+    def _set(name, value=1):
+        saved.setdefault(name, ops.get_option(name))
+        ops.set_option(name, value)
+
+    yield _set
+    for name, value in saved.items():
+        ops.set_option(name, value)

@@ -13,14 +13,16 @@ def test_qshift_tensor_ops_match_index_loops():
     g = load_golden("qshift_golden")["q"]
     y = ops.q_shift(torch.from_numpy(g["x"]), 1, 0.25, (3, 5)).numpy()
     assert np.array_equal(y, g["y"])
-    x = np.random.default_rng(0).standard_normal((2, 20, 22)).astype(np.float32)
-    assert np.array_equal(ops.q_shift(torch.from_numpy(x), 1, 0.25, (4, 5)).numpy(),
-                          qshift.q_shift_loops(x, 1, 0.25, (4, 5)))
+    for C in (22, 18, 6, 20):              # 22, 18, 6: unequal channel groups (C*gamma not an integer)
+        x = np.random.default_rng(C).standard_normal((2, 20, C)).astype(np.float32)
+        assert np.array_equal(ops.q_shift(torch.from_numpy(x), 1, 0.25, (4, 5)).numpy(),
+                              qshift.q_shift_loops(x, 1, 0.25, (4, 5))), C
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,Hp,Wp,C,dtype", [(2, 3, 5, 16, torch.float32), (2, 14, 14, 192, torch.float32),
-                                              (1, 7, 9, 22, torch.float32), (2, 24, 24, 1024, torch.bfloat16)])
+                                              (1, 7, 9, 22, torch.float32), (1, 7, 9, 20, torch.float32),
+                                              (2, 24, 24, 1024, torch.bfloat16)])
 def test_fused_qshift_mix_against_oracle(B, Hp, Wp, C, dtype):
     import vision_rwkv_amd as ops
     from oracle import qshift
@@ -210,11 +212,12 @@ def test_pos_embed_resize_restates_the_interpolation():
 @pytest.mark.gpu
 @pytest.mark.parametrize("N,dtype", [(1024, torch.bfloat16), (4096, torch.bfloat16), (768, torch.float32),
                                      (3072, torch.float32), (64, torch.float16), (8192, torch.bfloat16)])
-def test_row_fuse_against_tensor_ops(N, dtype):
-    """The fused row epilogues against the PyTorch-op sequence evaluated in fp32 on the same (rounded) inputs:
+def test_row_fuse_against_oracle(N, dtype):
+    """The fused row epilogues against the float64 row-by-row oracle (oracle/blocks.py) on the same (rounded) inputs:
     every pre / LayerNorm / post combination the blocks use, rows that do not fill a workgroup.
     Tolerance: 2e-3 of the row scale for fp32 I/O (fast exp / rcp in the gate), one 16-bit rounding otherwise."""
     import vision_rwkv_amd as ops
+    from oracle import blocks
     dev = "cuda:0"
     torch.manual_seed(N)
     rows = (3, 7)                                   # 21 rows: the last workgroup is partial
@@ -230,11 +233,15 @@ def test_row_fuse_against_tensor_ops(N, dtype):
         for gamma in ((g, None) if post == ops.ops.POST_RESIDUAL else (None,)):
             with torch.no_grad():
                 got = ops.row_fuse(a, o if post else None, w if ln else None, b if ln else None, gamma, pre, post)
-            f = lambda t: t.float() if t is not None else None
-            ref = ops.row_fuse_tensor_ops(f(a), f(o), f(w) if ln else None, f(b) if ln else None, f(gamma), pre, post)
+            f = lambda t: t.double().cpu().numpy() if t is not None else None
+            ref = blocks.row_epilogue(f(a), f(o), f(w) if ln else None, f(b) if ln else None, f(gamma), pre, post)
             assert got.dtype == dtype and got.shape == a.shape
-            err = (got.float() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-6)
+            err = np.abs(got.double().cpu().numpy() - ref).max() / max(np.abs(ref).max(), 1e-6)
             assert err <= tol, (pre, post, ln, gamma is not None, err)
+            # the tensor-op sequence the blocks fall back to is the same function
+            ft = lambda t: t.float() if t is not None else None
+            seq = ops.row_fuse_tensor_ops(ft(a), ft(o), ft(w) if ln else None, ft(b) if ln else None, ft(gamma), pre, post)
+            assert np.abs(seq.double().cpu().numpy() - ref).max() <= 2e-5 * max(np.abs(ref).max(), 1e-6)
     # a gradient is wanted: the tensor ops run and autograd works
     a2 = a.float().requires_grad_(True)
     ops.row_fuse(a2, o.float(), w.float(), b.float(), g.float(), ops.ops.PRE_NONE, ops.ops.POST_RESIDUAL).sum().backward()
@@ -244,11 +251,13 @@ def test_row_fuse_against_tensor_ops(N, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,T,C,dtype", [(2, 5, 64, torch.bfloat16), (3, 197, 768, torch.bfloat16), (1, 7, 128, torch.float16),
                                           (2, 9, 192, torch.float32)])
-def test_vrwkv6_mix_kernels_against_tensor_ops(B, T, C, dtype):
-    """maa_mix and groupnorm_gate against the tensor-op sequences evaluated in fp32 on the same (rounded) inputs.
+def test_vrwkv6_mix_kernels_against_oracle(B, T, C, dtype):
+    """maa_mix and groupnorm_gate against the float64 oracle (oracle/blocks.py) on the same (rounded) inputs.
     Tolerance: one 16-bit rounding of the result (1e-2 of the tensor's scale), 1e-5 for fp32 I/O."""
     import vision_rwkv_amd as ops
+    from oracle import blocks
     dev = "cuda:0"
+    f64 = lambda t: t.double().cpu().numpy()
     torch.manual_seed(C + T)
     x, sx = (torch.randn(B, T, C, device=dev).to(dtype) for _ in range(2))
     m = (0.3 * torch.randn(5, B, T, C, device=dev)).to(dtype)
@@ -256,9 +265,11 @@ def test_vrwkv6_mix_kernels_against_tensor_ops(B, T, C, dtype):
     tol = 1e-5 if dtype == torch.float32 else 1e-2
     with torch.no_grad():
         got = ops.maa_mix(x, sx, m, maas)
-    ref = ops.ops.maa_mix_tensor_ops(x.float(), sx.float(), m.float(), [a.float() for a in maas])
-    for g, r in zip(got, ref):
-        assert g.dtype == dtype and (g.float() - r).abs().max().item() <= tol * r.abs().max().item()
+    ref = blocks.maa_mix(f64(x), f64(sx), f64(m), [f64(a) for a in maas])
+    seq = ops.ops.maa_mix_tensor_ops(x.float(), sx.float(), m.float(), [a.float() for a in maas])
+    for g, r, sq in zip(got, ref, seq):
+        assert g.dtype == dtype and np.abs(f64(g) - r).max() <= tol * np.abs(r).max()
+        assert np.abs(f64(sq) - r).max() <= 1e-5 * np.abs(r).max()          # the tensor-op fallback is the same function
     if C % 64 == 0:
         H = C // 64
         for ydt in {torch.float32, dtype}:
@@ -267,9 +278,11 @@ def test_vrwkv6_mix_kernels_against_tensor_ops(B, T, C, dtype):
             w, b = torch.randn(C, device=dev).to(dtype), torch.randn(C, device=dev).to(dtype)
             with torch.no_grad():
                 got = ops.groupnorm_gate(y, gate, w, b, H)
-            ref = ops.ops.groupnorm_gate_tensor_ops(y.float(), gate.float(), w.float(), b.float(), H)
+            ref = blocks.groupnorm_gate(f64(y), f64(gate), f64(w), f64(b), H)
+            seq = ops.ops.groupnorm_gate_tensor_ops(y.float(), gate.float(), w.float(), b.float(), H)
             assert got.dtype == dtype and got.shape == gate.shape
-            assert (got.float() - ref).abs().max().item() <= tol * ref.abs().max().item()
+            assert np.abs(f64(got) - ref).max() <= tol * np.abs(ref).max()
+            assert np.abs(f64(seq) - ref).max() <= 1e-5 * np.abs(ref).max()
     # under autograd the tensor ops run
     xg = x.float().requires_grad_(True)
     sum(o.sum() for o in ops.maa_mix(xg, sx.float(), m.float(), [a.float() for a in maas])).backward()

@@ -88,9 +88,10 @@ def test_autograd_function_end_to_end(ops):
         assert rel_err(leaf.grad.cpu().numpy(), r) <= 2e-4
 
 
-def test_tiled_kernel_equals_sequential_kernel_full_size(ops, monkeypatch):
-    """VRWKV-B shape: the tiled kernel against the sequential one (forced through the environment), and
-    the sum identities that hold at any size."""
+def test_tiled_and_sequential_kernels_full_size(ops, force):
+    """VRWKV-B shape, random per-channel w, u: the tiled kernel and the sequential one (forced through the library
+    switch), each against the C oracle on every output, and the sum identities that hold at any size."""
+    from oracle import clib
     B, T, C = 64, 196, 768
     g = torch.Generator().manual_seed(5)
     k = torch.randn(B, T, C, generator=g).cuda()
@@ -99,18 +100,15 @@ def test_tiled_kernel_equals_sequential_kernel_full_size(ops, monkeypatch):
     w = ((torch.rand(C, generator=g) * 8 - 5) / T).cuda()
     u = (torch.rand(C, generator=g) - 0.5).cuda()
     got = ops.bi_wkv_backward(w, u, k, v, gy)
-    monkeypatch.setenv("VRWKV_BIWKV_BWD_PATH", "serial")
+    force("biwkv_bwd_serial")
     ref = ops.bi_wkv_backward(w, u, k, v, gy)
     torch.cuda.synchronize()
-    # two fp32 evaluations (the sequential one renormalises at every token and is the less accurate)
-    for a, b, name in zip(got, ref, ("gw", "gu", "gk", "gv")):
-        assert rel_err(a.cpu().numpy(), b.cpu().numpy()) <= 5e-4, name
-    # float64 closed form on a slice (gk, gv of a sequence depend on that sequence only)
-    from oracle import biwkv
-    sl = (slice(0, 2), slice(None), slice(640, 704))
     f = lambda x: x.cpu().numpy()
-    _, _, rk, rv = biwkv.biwkv_grads_closed(f(w[640:704]), f(u[640:704]), f(k[sl]), f(v[sl]), f(gy[sl]))
-    assert rel_err(f(got[2][sl]), rk) <= 1e-4 and rel_err(f(got[3][sl]), rv) <= 1e-4
+    want = clib.biwkv_bwd(f(w), f(u), f(k), f(v), f(gy))
+    for a, b, r, name in zip(got, ref, want, ("gw", "gu", "gk", "gv")):
+        assert rel_err(f(a), r) <= 1e-4, name
+        # the sequential kernel renormalises at every token and is the less accurate of the two
+        assert rel_err(f(b), r) <= 5e-4, name
     gk, gv = got[2], got[3]
     assert (gv.sum(1) - gy.sum(1)).abs().max().item() <= 1e-4 * gy.abs().sum(1).max().item()
     assert gk.sum(1).abs().max().item() <= 1e-4 * gk.abs().max().item() * T ** 0.5
@@ -140,7 +138,27 @@ def test_wave_scales_far_apart_and_sequence_lengths(ops, T):
     assert rel_err(gw, rw) <= 5e-4 and rel_err(gu, ru) <= 5e-4
 
 
-def test_long_sequence_tiled_equals_sequential(ops, monkeypatch):
+@pytest.mark.parametrize("T", [196, 500])
+def test_growing_weights_with_waves_far_apart(ops, T):
+    """Negative w with k = +40 on the first 28 tokens and -40 elsewhere (see the forward's test of that name):
+    finite, and equal to the oracle's gradients."""
+    from oracle import clib
+    B, C = 2, 64
+    rng = np.random.default_rng(T + 1)
+    k = np.full((B, T, C), -40.0, np.float32)
+    k[:, :28] = 40.0
+    k += rng.standard_normal((B, T, C)).astype(np.float32)
+    v, gy = (rng.standard_normal((B, T, C)).astype(np.float32) for _ in range(2))
+    w = (np.array([-0.13, -0.05, -0.02, 0.02] * (C // 4)) * 196.0 / T).astype(np.float32)
+    u = np.zeros(C, np.float32)
+    gw, gu, gk, gv, *_ = run(ops, w, u, k, v, gy)
+    ref = clib.biwkv_bwd(w, u, k, v, gy)
+    for got, want, name in zip((gw, gu, gk, gv), ref, ("gw", "gu", "gk", "gv")):
+        assert np.isfinite(got).all(), name
+        assert rel_err(got, want) <= 5e-4, name
+
+
+def test_long_sequence_tiled_equals_sequential(ops, force):
     """VRWKV-L at 384x384 (T = 576, three super-chunks): the three-launch tiled path against the sequential
     kernel, the float64 closed form on a slice, and the sum identities."""
     B, T, C = 4, 576, 256
@@ -151,7 +169,7 @@ def test_long_sequence_tiled_equals_sequential(ops, monkeypatch):
     w = ((torch.rand(C, generator=g) * 8 - 5) / T).cuda()
     u = (torch.rand(C, generator=g) - 0.5).cuda()
     got = ops.bi_wkv_backward(w, u, k, v, gy)
-    monkeypatch.setenv("VRWKV_BIWKV_BWD_PATH", "serial")
+    force("biwkv_bwd_serial")
     ref = ops.bi_wkv_backward(w, u, k, v, gy)
     torch.cuda.synchronize()
     for a, b, name in zip(got, ref, ("gw", "gu", "gk", "gv")):

@@ -134,7 +134,7 @@ def test_two_and_three_super_chunks_16bit(ops, B, T, C, dtype):
     assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= TOL_16
 
 
-def test_one_launch_and_two_kernel_paths_agree(ops, monkeypatch):
+def test_one_launch_and_two_kernel_paths_agree(ops, force):
     """The same 16-bit sequence through the one-launch kernel and through the aggregate + emit kernels: both round
     the same fp32 arithmetic to bf16, so they may differ by an output ulp here and there, no more."""
     B, T, C = 4, 576, 256
@@ -143,7 +143,7 @@ def test_one_launch_and_two_kernel_paths_agree(ops, monkeypatch):
     v = rng.standard_normal((B, T, C), dtype=np.float32)
     w, u = baseline_wu(C, T)
     y1, _, _ = run(ops, w, u, k, v, torch.bfloat16)
-    monkeypatch.setenv("VRWKV_BIWKV_NO_RESIDENT", "1")
+    force("biwkv_no_resident")
     y2, _, _ = run(ops, w, u, k, v, torch.bfloat16)
     assert np.abs(y1 - y2).max() <= 2.0 ** -7 * np.abs(y2).max()
     assert (y1 != y2).mean() < 0.02
@@ -196,6 +196,26 @@ def test_huge_k_range_stays_finite(ops):
     y, _, _ = run(ops, w, u, k, v)
     assert np.isfinite(y).all()
     assert rel_err(y, clib.biwkv_fwd(w, u, k, v)) <= TOL_F32
+
+
+@pytest.mark.parametrize("T,dtype", [(196, torch.float32), (196, torch.bfloat16), (576, torch.bfloat16), (900, torch.float32)])
+def test_growing_weights_with_waves_far_apart_stay_finite(ops, T, dtype):
+    """Negative w (weights that grow with distance) together with k = +40 on the first 28 tokens and -40 elsewhere:
+    the carried sums grow by up to e^{|w| T} while the light waves raise them by 2^115 to their own scale.  Channels:
+    w = -0.13 (growth 2^37 at T=196: the renormalising path), w = -0.05 and -0.02 (plain sums, growth 2^14 / 2^6),
+    w = +0.02, and the same spread scaled to the longer sequences."""
+    from oracle import clib
+    B, C = 2, 64
+    rng = np.random.default_rng(T)
+    k = np.full((B, T, C), -40.0, np.float32)
+    k[:, :28] = 40.0
+    k += rng.standard_normal((B, T, C)).astype(np.float32)
+    v = rng.standard_normal((B, T, C), dtype=np.float32)
+    w = (np.array([-0.13, -0.05, -0.02, 0.02] * (C // 4)) * 196.0 / T).astype(np.float32)
+    u = np.zeros(C, np.float32)
+    y, kr, vr = run(ops, w, u, k, v, dtype)
+    assert np.isfinite(y).all()
+    assert rel_err(y, clib.biwkv_fwd(w, u, kr, vr)) <= (TOL_F32 if dtype == torch.float32 else 1e-2)
 
 
 def test_properties_at_full_size(ops):

@@ -1,0 +1,205 @@
+"""Parity at the benchmark configurations' own shapes and dtypes, every output against the C / float64 oracle:
+  config 1 / 3   backward of both operators at B=64, T=196, C=768 (all five / four outputs incl. the batch-reduced
+                 gw, gu), against oracle/c (brute-force softmax form for Bi-WKV, adjoint recurrence for wkv6);
+  config 4       Bi-WKV forward at B=32, T=576, C=1024 in bf16 and fp32, its backward at that T and C, and two
+                 VRWKV-L blocks (C=1024, hidden 4096, key_norm, post-norm, layer scale 1e-5, 12x12 -> 24x24 position
+                 table) in bf16: fused kernels against the tensor-op path, and against a float32 CPU evaluation of the
+                 same blocks with the oracle's Bi-WKV inside.
+Error measure: max|x - ref| / max(|ref|, rms(ref)) (conftest.rel_err)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import vision_rwkv_amd
+    assert torch.cuda.is_available()
+    return vision_rwkv_amd
+
+
+def baseline_wu(C, T):
+    c = np.arange(C)
+    w = ((-5.0 + 8.0 * c / (C - 1)) / T).astype(np.float32)
+    u = ((np.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T).astype(np.float32)
+    return w, u
+
+
+def test_biwkv_backward_config1_every_output_against_the_oracle(ops):
+    """B=64, T=196, C=768, fp32: gk, gv and the sums gw, gu over 12 544 (batch, token) pairs.
+    Tolerance 1e-4 for all four (measured: gk 1.8e-5, gv 1.3e-5, gw 3e-6, gu 1.6e-6; gw, gu are sums of 12 544 signed
+    fp32 terms, partial sums per tile, then a fixed-order reduction)."""
+    from oracle import clib
+    B, T, C = 64, 196, 768
+    rng = np.random.default_rng(5)
+    k, v, gy = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(3))
+    w, u = baseline_wu(C, T)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    got = [x.cpu().numpy() for x in ops.bi_wkv_backward(t(w), t(u), t(k), t(v), t(gy))]
+    ref = clib.biwkv_bwd(w, u, k, v, gy)
+    errs = {n: rel_err(g, r) for g, r, n in zip(got, ref, ("gw", "gu", "gk", "gv"))}
+    print("biwkv bwd config 1 fp32:", errs)
+    assert max(errs.values()) <= 1e-4, errs
+
+
+def test_biwkv_backward_config1_bf16_io(ops):
+    """Same shape, bf16 k, v, gy (reference on the rounded inputs): gk, gv carry one bf16 rounding of the result."""
+    from oracle import clib
+    B, T, C = 64, 196, 768
+    rng = np.random.default_rng(6)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    k, v, gy = (t(rng.standard_normal((B, T, C), dtype=np.float32)).bfloat16() for _ in range(3))
+    w, u = baseline_wu(C, T)
+    got = [x.float().cpu().numpy() for x in ops.bi_wkv_backward(t(w), t(u), k, v, gy)]
+    f = lambda x: x.float().cpu().numpy()
+    ref = clib.biwkv_bwd(w, u, f(k), f(v), f(gy))
+    errs = {n: rel_err(g, r) for g, r, n in zip(got, ref, ("gw", "gu", "gk", "gv"))}
+    print("biwkv bwd config 1 bf16:", errs)
+    assert errs["gk"] <= 1e-2 and errs["gv"] <= 1e-2          # one bf16 rounding of the result: 2^-8
+    assert errs["gw"] <= 1e-4 and errs["gu"] <= 1e-4          # fp32 outputs of fp32 sums
+
+
+def test_wkv6_backward_config3_every_output_against_the_oracle(ops):
+    """B=64, T=196, C=768, H=12, bf16 r, k, v, fp32 decay logit and gy: gr, gk, gv, gw, gu against the float64 adjoint
+    recurrence.  Tolerance 1e-3 (the operator's forward tolerance) for gr, gk, gv, gu (measured 5e-5, 5e-5, 9e-5,
+    1.2e-5).  gw: 2e-3 -- it is ld_n times a running difference sum(a - b) of two sums that nearly cancel, formed from
+    products of head + tail bf16 operands; its worst element over 9.6 M measures 1.5e-3 of the tensor's rms."""
+    from oracle import clib
+    B, T, H = 64, 196, 12
+    C = H * 64
+    g = torch.Generator().manual_seed(21)
+    r, k, v = (torch.randn(B, T, C, generator=g).bfloat16() for _ in range(3))
+    w = torch.randn(B, T, C, generator=g) * 0.5 - 0.5
+    u = torch.randn(H, 64, generator=g) * 0.1
+    gy = torch.randn(B, T, C, generator=g)
+    got = ops.wkv6_backward(B, T, C, H, r.to(DEV), k.to(DEV), v.to(DEV), w.to(DEV), u.to(DEV), gy.to(DEV))
+    got = [x.cpu().numpy() for x in got]
+    f = lambda x: x.float().numpy()
+    ref = clib.wkv6_bwd(f(r), f(k), f(v), f(w), f(u), f(gy), H)
+    errs = {n: rel_err(a, b) for a, b, n in zip(got, ref, ("gr", "gk", "gv", "gw", "gu"))}
+    print("wkv6 bwd config 3:", errs)
+    for n in ("gr", "gk", "gv", "gu"):
+        assert errs[n] <= 1e-3, (n, errs)
+    assert errs["gw"] <= 2e-3, errs
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 1e-2), (torch.float32, 1e-4)])
+def test_biwkv_forward_config4_layer_shape(ops, dtype, tol):
+    """B=32, T=576, C=1024: the shape every VRWKV-L layer calls the operator with (bf16: the one-launch kernel for
+    three super-chunks; fp32: the two-kernel long-sequence path)."""
+    from oracle import clib
+    B, T, C = 32, 576, 1024
+    rng = np.random.default_rng(44)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    k, v = (t(rng.standard_normal((B, T, C), dtype=np.float32)).to(dtype) for _ in range(2))
+    w, u = baseline_wu(C, T)
+    y = ops.bi_wkv_forward(t(w), t(u), k, v)
+    assert y.dtype == dtype
+    f = lambda x: x.float().cpu().numpy()
+    ref = clib.biwkv_fwd(w, u, f(k), f(v))
+    err = rel_err(f(y), ref)
+    print("biwkv fwd config-4 layer shape", dtype, err)
+    assert err <= tol
+
+
+def test_biwkv_backward_config4_layer_shape(ops):
+    """T=576, C=1024 (three-launch long-sequence backward), batch 8 so that the O(T^2) oracle stays in seconds."""
+    from oracle import clib
+    B, T, C = 8, 576, 1024
+    rng = np.random.default_rng(45)
+    k, v, gy = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(3))
+    w, u = baseline_wu(C, T)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    got = [x.cpu().numpy() for x in ops.bi_wkv_backward(t(w), t(u), t(k), t(v), t(gy))]
+    ref = clib.biwkv_bwd(w, u, k, v, gy)
+    errs = {n: rel_err(g, r) for g, r, n in zip(got, ref, ("gw", "gu", "gk", "gv"))}
+    print("biwkv bwd T=576 C=1024:", errs)
+    assert max(errs.values()) <= 1e-4, errs
+
+
+def _record_branches(net, store):
+    hooks = []
+    for i, blk in enumerate(net.layers):
+        hooks.append(blk.att.register_forward_hook(lambda m, a, out, i=i: store.__setitem__(f"att{i}", out.detach().float().cpu())))
+        hooks.append(blk.ffn.register_forward_hook(lambda m, a, out, i=i: store.__setitem__(f"ffn{i}", out.detach().float().cpu())))
+        hooks.append(blk.att.key.register_forward_hook(lambda m, a, out, i=i: store.__setitem__(f"k{i}", out.detach().cpu())))
+        hooks.append(blk.att.value.register_forward_hook(lambda m, a, out, i=i: store.__setitem__(f"v{i}", out.detach().cpu())))
+    return hooks
+
+
+def test_vrwkv_l_blocks_bf16_fused_eager_and_oracle(ops, monkeypatch):
+    """Two VRWKV-L blocks at 384x384 (T=576, C=1024, hidden 4096, key_norm, post-norm, layer scale 1e-5, position
+    table 12x12 -> 24x24) in bf16.  With a layer scale of 1e-5 the model output hardly sees the branches, so the
+    branch outputs (att, ffn of each block) are compared as well.
+      fused vs tensor-op path, both bf16 on the GPU: a few bf16 roundings apart;
+      fused vs float32 CPU evaluation with the oracle's Bi-WKV: the bf16 GEMM chain's rounding (inputs 2^-9 each);
+      the operator itself on the k, v the first block produced, against the oracle at bf16 tolerance."""
+    from oracle import clib
+    import vision_rwkv_amd.backbone as bb
+    torch.manual_seed(4)
+    net32 = ops.vrwkv_l(depth=2).eval()
+    with torch.no_grad():
+        net32.pos_embed.normal_(0, 0.02)
+        for blk in net32.layers:                      # parameters away from their 1 / 0 defaults
+            for ln in (blk.ln1, blk.ln2, blk.att.key_norm, blk.ffn.key_norm):
+                ln.weight.uniform_(0.5, 1.5)
+                ln.bias.normal_(0, 0.1)
+    img = torch.randn(2, 3, 384, 384)
+    net16 = copy.deepcopy(net32).to(DEV).bfloat16()
+    # the float32 CPU reference runs the same modules on the bf16-rounded weights
+    net32.load_state_dict({k: v.float().cpu() for k, v in net16.state_dict().items()})
+
+    fused, eager, cpu = {}, {}, {}
+    with torch.no_grad():
+        hooks = _record_branches(net16, fused)
+        y_fused = net16(img.to(DEV).bfloat16()).float().cpu()
+        for h in hooks:
+            h.remove()
+        hooks = _record_branches(net16, eager)
+        for m in net16.modules():
+            if hasattr(m, "fused_shift"):
+                m.fused_shift = False
+        monkeypatch.setattr(ops.ops, "ROW_FUSE_ENABLED", False)
+        y_eager = net16(img.to(DEV).bfloat16()).float().cpu()
+        for h in hooks:
+            h.remove()
+
+        # float32 on the CPU with the oracle operator inside (nothing of the HIP library runs here)
+        def oracle_wkv(w, u, k, v):
+            y = clib.biwkv_fwd(w.float().numpy(), u.float().numpy(), k.float().numpy(), v.float().numpy())
+            return torch.from_numpy(y).float()
+        monkeypatch.setattr(bb, "RUN_CUDA", oracle_wkv)
+        monkeypatch.setattr(bb, "bi_wkv_forward", oracle_wkv)
+        for m in net32.modules():
+            if hasattr(m, "fused_shift"):
+                m.fused_shift = False
+        hooks = _record_branches(net32, cpu)
+        y_cpu = net32(img.bfloat16().float())
+        for h in hooks:
+            h.remove()
+
+    assert tuple(y_fused.shape) == (2, 1024, 24, 24)
+    errs = {"out_eager": rel_err(y_fused.numpy(), y_eager.numpy()), "out_cpu": rel_err(y_fused.numpy(), y_cpu.numpy())}
+    for name in ("att0", "ffn0", "att1", "ffn1"):
+        errs[name + "_eager"] = rel_err(fused[name].numpy(), eager[name].numpy())
+        errs[name + "_cpu"] = rel_err(fused[name].numpy(), cpu[name].numpy())
+    print("VRWKV-L blocks bf16:", {k: round(v, 5) for k, v in errs.items()})
+    for name, e in errs.items():
+        assert e <= 6e-2, (name, errs)
+    # the operator on this block's own k, v (bf16, T=576, C=1024)
+    att = net16.layers[0].att
+    k, v = fused["k0"].to(DEV), fused["v0"].to(DEV)
+    T = k.shape[1]
+    with torch.no_grad():
+        y = ops.RUN_CUDA(att.spatial_decay / T, att.spatial_first / T, k, v)
+    assert y.dtype == torch.bfloat16
+    ref = clib.biwkv_fwd((att.spatial_decay / T).detach().float().cpu().numpy(),
+                         (att.spatial_first / T).detach().float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy())
+    assert rel_err(y.float().cpu().numpy(), ref) <= 1e-2

@@ -80,11 +80,11 @@ def test_extreme_decay(ops, w_mean):
     assert rel_err(y, clib.wkv6_fwd(r, k, v, w, u, 2)) <= TOL
 
 
-def test_chunked_and_sequential_kernels_agree(ops, monkeypatch):
+def test_chunked_and_sequential_kernels_agree(ops, force):
     """The matrix-core path and the sequential-state path are independent implementations."""
     r, k, v, w, u = gen(3, 196, 2, 21)
     y_chunk, *_ = run(ops, r, k, v, w, u, 2, torch.bfloat16)
-    monkeypatch.setenv("VRWKV_WKV6_PATH", "scalar")
+    force("wkv6_fwd_scalar")
     y_seq, *_ = run(ops, r, k, v, w, u, 2, torch.bfloat16)
     assert rel_err(y_chunk, y_seq) <= TOL
 

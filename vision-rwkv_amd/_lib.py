@@ -43,6 +43,10 @@ def _declare(lib):
     lib.vrwkv_version.restype = i
     lib.vrwkv_last_error.argtypes = []
     lib.vrwkv_last_error.restype = c.c_char_p
+    lib.vrwkv_set_option.argtypes = [c.c_char_p, i]
+    lib.vrwkv_set_option.restype = i
+    lib.vrwkv_get_option.argtypes = [c.c_char_p, c.POINTER(c.c_int)]
+    lib.vrwkv_get_option.restype = i
     lib.vrwkv_biwkv_fwd_workspace_bytes.argtypes = [i, i, i, i]
     lib.vrwkv_biwkv_fwd_workspace_bytes.restype = sz
     lib.vrwkv_biwkv_fwd.argtypes = [fp, fp, vp, vp, vp, i, i, i, i, vp, sz, vp]
@@ -95,6 +99,33 @@ def lib():
                 "or make -C vision-rwkv_amd/csrc); there is no non-HIP fallback")
         _lib = _declare(ctypes.CDLL(LIB_PATH))
     return _lib
+
+
+def get_option(name):
+    """Value of a tuning / testing switch of the library (include/vrwkv_hip.h lists the names)."""
+    out = ctypes.c_int(0)
+    check(lib().vrwkv_get_option(name.encode(), ctypes.byref(out)))
+    return out.value
+
+
+def set_option(name, value):
+    check(lib().vrwkv_set_option(name.encode(), int(value)))
+
+
+class option:
+    """with option("wkv6_fwd_scalar", 1): ...  -- sets a switch for the block and restores it afterwards."""
+
+    def __init__(self, name, value):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        self.old = get_option(self.name)
+        set_option(self.name, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        set_option(self.name, self.old)
+        return False
 
 
 def check(status):

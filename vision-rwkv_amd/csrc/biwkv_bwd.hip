@@ -64,8 +64,7 @@ struct BwdPlan {
 BwdPlan make_bwd_plan(int B, int T, int C) {
     BwdPlan p;
     static const int kL[] = {4, 8, 16, 28};
-    const char* path = getenv("VRWKV_BIWKV_BWD_PATH");       // "serial" forces the sequential kernel (testing)
-    const bool tiled = !(path && path[0] == 's') && (long long)T * C < (1LL << 29);
+    const bool tiled = !option(OPT_BIWKV_BWD_SERIAL) && (long long)T * C < (1LL << 29);   // the option forces the sequential kernel (testing)
     if (tiled) {
         for (int i = 3; i >= 0; --i)
             if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX) p.L = kL[i];     // smallest L that fits: most waves per tile
@@ -98,8 +97,7 @@ void launch_tiled(const BwdPlan& p, const float* w, const float* u, const IO* k,
     if (p.nSC == 1) {
         if constexpr (sizeof(IO) == 4 && L % 4 == 0) {
             const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
-            const char* ns = getenv("VRWKV_BIWKV_NO_STAGE");
-            if (aligned && !(ns && atoi(ns))) {
+            if (aligned && !option(OPT_BIWKV_NO_STAGE)) {
                 hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 0, true>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
                                    gw_part, gu_part, B, T, C, geo);
                 return;

@@ -22,11 +22,11 @@
 // ascending sweep (past side) -> descending sweep (future side).
 //
 // Scaling: as in the forward's plain-sum path every wave works in units of 2^Rw, Rw = ceil(max kappa)
-// over its tokens, and z carries 2^-Re with Re = max(Rw, R - 100) the scale its denominators were
+// over its tokens, and z carries 2^-Re with Re = max(Rw, R - plain_sum_up_cap) the scale its denominators were
 // actually formed at.  Another wave's z-aggregates are brought over with the exact factor
 // 2^(Rw_mine - Re_theirs): that is the same power of two by which my E entered their denominators, so
 // the product stays below |gy| 2^41 and nothing overflows.  Tiles outside the plain-sum regime
-// (|omega| (T+1) + |mu| > 40) are left to the sequential kernel, which renormalises at every token.
+// (outside_plain_sum) are left to the sequential kernel, which renormalises at every token.
 #pragma once
 #include "biwkv_fwd_impl.h"
 #include "biwkv_bwd_serial.h"
@@ -54,7 +54,7 @@ __device__ __forceinline__ void store1(__amdgpu_buffer_rsrc_t r, unsigned voff, 
 
 // True when this wave's 64 channels may use the plain-sum path (wave-uniform).
 __device__ __forceinline__ bool bwd_tile_is_fast(float om, float mu, int T) {
-    const bool bad = !(fabsf(om) * (float)(T + 1) + fabsf(mu) <= FAST_LIMIT);
+    const bool bad = outside_plain_sum(om, mu, T);
     return __builtin_amdgcn_ballot_w64(bad) == 0ull;
 }
 
@@ -153,6 +153,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // the skipped tile's rows must have landed
                 issue_stage(next_tile);
             }
+            wg_barrier();                                     // keeps the LDS reuse order of the computed tiles around it
             continue;
         }
         const int cc = cok ? c0 : 0;                         // in-range column for the auxiliary table
@@ -268,6 +269,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
 
         const float gd = fast_exp2(-om), cu = fast_exp2(mu);
         const float G = fast_exp2(-om * (float)L);
+        const float up_cap = floorf(plain_sum_up_cap(om, T));
 
         // ------------------------------ phase 1: the forward ------------------------------
         float E[L], V[L];
@@ -355,7 +357,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
                     d = fmaf(G, d, ldexpf(ld[s], sh));
                 }
             Rw_to_R = r - Rw;
-            const float upf = fminf(r - Rw, 100.f);
+            const float upf = fminf(r - Rw, up_cap);
             const int up = (int)upf;
             a = ldexpf(a, up); bb = ldexpf(bb, up); c = ldexpf(c, up); d = ldexpf(d, up);
             Re = r - upf;                                     // the scale the carried terms really have
@@ -398,7 +400,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             s2[wave][8][lane] = Re;
             wg_barrier();
             if (wave == 0 && cok) {
-                const float Rg = Re + fminf(Rw_to_R, 100.f);                  // = R (Re = R - min(R - Rw, 100))
+                const float Rg = Re + fminf(Rw_to_R, up_cap);                 // = R (Re = R - min(R - Rw, up_cap))
                 ZScan ps, fs;
                 const float nL = (float)L;
                 for (int sw = 0; sw < S; ++sw) {

@@ -26,13 +26,16 @@
 //
 // Two code paths, chosen per tile from (w, u, T) alone and therefore identically by
 // every wave that touches a channel tile:
-//   fast   |omega|*(T+1) + |mu| <= 40.  Each wave uses its own integer reference exponent
+//   fast   |omega|*(T+1) + |mu| <= 40, and for negative omega (weights that grow with distance) |omega|*(T+1) <= 16.
+//          Each wave uses its own integer reference exponent
 //          Rw = ceil(max kappa) over its tokens; E_t = 2^(kappa_t-Rw) <= 1 is computed once per
 //          token and reused by both directions and both phases; states are plain decayed sums
 //          a <- g*a + E_t v_t (g = 2^-omega), no per-token max.  Waves exchange their chunk
-//          aggregates once per tile and rescale each other's by exact powers of two.  Under the
-//          bound every state stays within 2^+-41 of the largest term, so nothing overflows, and a
-//          term that underflows is below 2^-80 of its denominator.
+//          aggregates once per tile and rescale each other's by exact powers of two.  A carried sum is at
+//          most T * 2^growth (growth = max(0, -omega) (T+1) <= 16) in units of the largest wave scale, and the
+//          shift that brings it to a wave's own scale is capped (plain_sum_up_cap) so that it stays below
+//          2^96 |v|: nothing overflows, and a term that the cap or an underflow drops is below 2^-27 of its
+//          denominator.
 //   robust anything else: every state is a (num, den, exponent) triple renormalised at
 //          every token, exactly the reference's recurrence, for both directions; those tiles
 //          are done in a second walk after the fast ones.
@@ -43,6 +46,20 @@ namespace vrwkv {
 namespace biwkv_fwd_detail {
 
 constexpr float FAST_LIMIT = 40.0f;
+constexpr float GROW_LIMIT = 16.0f;
+
+// True when a channel is outside the plain-sum regime (log2 units: om = w log2e, mu = u log2e).
+__device__ __forceinline__ bool outside_plain_sum(float om, float mu, int T) {
+    const float span = fabsf(om) * (float)(T + 1);
+    return !(span + fabsf(mu) <= FAST_LIMIT) || (om < 0.f && span > GROW_LIMIT);
+}
+// Upper limit of the exponent by which a carried sum is raised from the common scale 2^R to a wave's own scale
+// 2^Rw: the sum is at most T 2^growth |v| in units of 2^R, so below 2^96 |v| afterwards.  Past the limit the wave's
+// own terms are negligible against the carry (the carry has decayed by at most 2^-40), so the limit only keeps
+// fp32 finite.
+__device__ __forceinline__ float plain_sum_up_cap(float om, int T) {
+    return 96.f - fmaxf(-om, 0.f) * (float)(T + 1) - __builtin_amdgcn_logf((float)T);
+}
 constexpr int NSLOT = 6;   // workspace floats per (b, super-chunk, channel): A, B, pA|R, Cg, D, pC
 
 // Waves per workgroup: at most 8, i.e. two per SIMD, which leaves every wave 256 VGPRs -- enough
@@ -209,7 +226,7 @@ struct BiwkvTile {
         for (int e = 0; e < VEC; ++e) {
             om[e] = wu.w[e] * LOG2E;
             mu[e] = wu.u[e] * LOG2E;
-            bad = bad || !(fabsf(om[e]) * (float)(T + 1) + fabsf(mu[e]) <= FAST_LIMIT);
+            bad = bad || outside_plain_sum(om[e], mu[e], T);
         }
         return __builtin_amdgcn_ballot_w64(bad) != 0ull;
     }
@@ -218,8 +235,9 @@ struct BiwkvTile {
     // consumed) issues the loads of `next` into Kn, Vn when next < n_tiles.  Tiles that need
     // the robust path are skipped here and handled by run_robust() afterwards.
     // Consecutive tiles alternate between the two LDS buffers (`par`), so one barrier per
-    // exchange is enough: a wave can only write buffer `par` again after passing a barrier of
-    // the tile in between, which every wave reaches after its last read of this tile.
+    // exchange is enough: a wave can only write buffer `par` again after passing the barrier of
+    // the tile in between (a skipped tile has one too), which every wave reaches after its last
+    // read of this tile.
     __device__ __forceinline__ void run(int tile, int next, int par, P (&K)[L], P (&V)[L], const WU& wu,
                                         P (&Kn)[L], P (&Vn)[L], WU& wun) const {
         const Where q = locate(tile);
@@ -230,6 +248,8 @@ struct BiwkvTile {
 
         float om[VEC], mu[VEC];
         if (tile_is_robust(wu, om, mu)) {
+            // workgroup-uniform branch; the barrier stands in for the exchange barrier of a computed tile
+            if (STAGED) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); else lds_barrier();
             if (next < g.n_tiles) {
                 if (STAGED) {
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the skipped tile's rows must have landed
@@ -350,8 +370,7 @@ struct BiwkvTile {
         //  3. R = max Rw.  All Rw are integers, so bringing another wave's aggregate to the common
         //     scale is an exact ldexp (no exponential); the carry-in is accumulated at scale 2^R
         //     and then shifted to the wave's own scale 2^Rw, in which the sweeps run unchanged
-        //     (y is a ratio, the scale cancels).  The shift is capped at 2^100: beyond that the
-        //     wave's own terms are below 2^-60 of the carry and the cap only keeps fp32 finite.
+        //     (y is a ratio, the scale cancels).  The shift is capped (plain_sum_up_cap).
         float gd[VEC], Rw[VEC], Rpub[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -461,7 +480,7 @@ struct BiwkvTile {
                         ad = fmaf(G[e], ad, ldexpf(ld[s], sh));
                     }
                 // to the wave's own scale
-                const int up = (int)fminf(r - Rw[e], 100.f);
+                const int up = (int)fminf(r - Rw[e], plain_sum_up_cap(om[e], T));
                 aa = ldexpf(aa, up); ab = ldexpf(ab, up); ac = ldexpf(ac, up); ad = ldexpf(ad, up);
             }
             a[e] = aa; bb[e] = ab; c[e] = ac; d[e] = ad;
@@ -727,11 +746,6 @@ struct Plan {
 constexpr int kLs[] = {4, 8, 16, 28};
 constexpr int kNumL = sizeof(kLs) / sizeof(kLs[0]);
 
-inline int env_int(const char* name) {
-    const char* s = getenv(name);
-    return s ? atoi(s) : 0;
-}
-
 inline int num_cus() {
     static int n = 0;
     if (n == 0) {
@@ -747,8 +761,8 @@ inline int num_cus() {
 inline Plan make_plan(int B, int T, int C, int io_dtype) {
     Plan p;
     (void)io_dtype;
-    const int el = env_int("VRWKV_BIWKV_L");              // tuning overrides
-    const int es = env_int("VRWKV_BIWKV_S");
+    const int el = option(OPT_BIWKV_L);              // tuning overrides
+    const int es = option(OPT_BIWKV_S);
     p.VEC = 1;
     int best = -1, best_waste = 1 << 30;
     for (int i = 0; i < kNumL; ++i) {
@@ -777,7 +791,7 @@ inline Plan make_plan(int B, int T, int C, int io_dtype) {
     // persistent grid: as many workgroups as can be resident at once
     const int wg_per_cu = (cap / p.S) > 0 ? (cap / p.S) : 1;
     int grid = num_cus() * wg_per_cu;
-    const int eg = env_int("VRWKV_BIWKV_GRID");
+    const int eg = option(OPT_BIWKV_GRID);
     if (eg > 0) grid = eg;
     p.grid = grid < p.geom.n_tiles ? grid : p.geom.n_tiles;
     return p;
@@ -794,14 +808,14 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
     // fp32 rows are staged through LDS in 16-byte pieces when the layout allows it
     if constexpr (VEC == 1) {
         const bool aligned = C % (16 / (int)sizeof(IO)) == 0 && (((uintptr_t)k | (uintptr_t)v | (uintptr_t)y) & 15) == 0;
-        if (aligned && !env_int("VRWKV_BIWKV_NO_STAGE")) {
+        if (aligned && !option(OPT_BIWKV_NO_STAGE)) {
             if (!p.multi()) {
                 hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
-            } else if (sizeof(IO) == 2 && L == 28 && p.nSC <= 3 && !env_int("VRWKV_BIWKV_NO_RESIDENT")) {
+            } else if (sizeof(IO) == 2 && L == 28 && p.nSC <= 3 && !option(OPT_BIWKV_NO_RESIDENT)) {
                 // two or three super-chunks of 16-bit rows fit a workgroup's registers: one launch, k and v read once
                 if constexpr (sizeof(IO) == 2 && L == 28) {
                     const int n_seq = B * p.geom.n_ctile;
-                    const int eg = env_int("VRWKV_BIWKV_GRID");
+                    const int eg = option(OPT_BIWKV_GRID);
                     const int g1 = eg > 0 ? eg : num_cus();
                     const dim3 rgrid(g1 < n_seq ? g1 : n_seq);
                     const bool short_chunks = T <= p.nSC * 8 * 24;        // 24-token chunks need no spills with three super-chunks

@@ -200,7 +200,7 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
         const bool cok = c0 < C;
         const float wv = cok ? w_[c0] : 0.f, uv = cok ? u_[c0] : 0.f;
         const float om = wv * LOG2E, mu = uv * LOG2E;
-        const bool bad = !(fabsf(om) * (float)(T + 1) + fabsf(mu) <= FAST_LIMIT);
+        const bool bad = outside_plain_sum(om, mu, T);
         if (__builtin_amdgcn_ballot_w64(bad) != 0ull) {
             // outside the plain-sum regime: the renormalising recurrence, super-chunk aggregates through the workspace
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");              // the rows already on their way must land first
@@ -349,7 +349,7 @@ void biwkv_fwd_resident_kernel(const float* __restrict__ w_, const float* __rest
                 }
             const float r = fmaxf(Rs[sc], fmaxf(r1, r2));
             const int s0 = shift_of(Rs[sc], r), s1 = shift_of(r1, r), s2_ = shift_of(r2, r);
-            const int up = (int)fminf(r - Rw[sc], 100.f);                 // to the wave's own scale
+            const int up = (int)fminf(r - Rw[sc], plain_sum_up_cap(om, T));   // to the wave's own scale
             fa[sc] = ldexpf(fmaf(Gpre, ldexpf(ca, s1), ldexpf(ia[sc], s0)), up);
             fb[sc] = ldexpf(fmaf(Gpre, ldexpf(cb, s1), ldexpf(ib[sc], s0)), up);
             fc[sc] = ldexpf(fmaf(Gpost, ldexpf(cc, s2_), ldexpf(ic[sc], s0)), up);

@@ -14,6 +14,22 @@ void set_error(const char* fmt, ...);
 // Returns VRWKV_OK, or VRWKV_LAUNCH_FAILED after recording hipGetLastError()'s text.
 int check_launch(const char* what);
 
+// Tuning / testing switches (0 = default behaviour).  Their initial values come from the environment variables
+// VRWKV_<NAME IN CAPITALS>, read once per process; vrwkv_set_option changes them afterwards.
+enum Option {
+    OPT_BIWKV_L,            // tokens per wave of the Bi-WKV forward (4, 8, 16, 28)
+    OPT_BIWKV_S,            // waves per workgroup on the long-sequence path
+    OPT_BIWKV_GRID,         // persistent grid size
+    OPT_BIWKV_NO_STAGE,     // register loads instead of LDS-staged rows
+    OPT_BIWKV_NO_RESIDENT,  // two-kernel long-sequence path also where the one-launch kernel applies
+    OPT_BIWKV_BWD_SERIAL,   // sequential Bi-WKV backward kernel
+    OPT_WKV6_FWD_SCALAR,    // sequential-state wkv6 forward kernel
+    OPT_WKV6_BWD_SCALAR,    // sequential wkv6 backward sweeps
+    OPT_WKV6_BWD_UNFUSED,   // one launch per wkv6 backward scan
+    N_OPTIONS
+};
+int option(Option o);
+
 constexpr int WAVE = 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float NEG_BIG = -1e38f;   // "empty state" exponent, bi_wkv_kernel.cu:14

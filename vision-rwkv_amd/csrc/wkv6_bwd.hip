@@ -242,6 +242,11 @@ void wkv6_bwd_fallback(const IO* r_, const IO* k_, const IO* v_, const WT* w_, c
     wkv6_bwd_sweep_v_body<IO, WT, 0, W_IS_EW>(bh, r_, k_, w_, u_, gy_, gv_, T, C, H);
 }
 
+__global__ void clear_flags_kernel(unsigned char* flags, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) flags[i] = 0;
+}
+
 template <typename IO, typename WT, bool EW>
 int launch_all(const void* r, const void* k, const void* v, const void* w, const float* u, const float* gy,
                float* gr, float* gk, float* gv, float* gw, float* gu, float* ws, int B, int T, int C, int H, hipStream_t st) {
@@ -253,11 +258,11 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
     float* gu_part = ws + (size_t)B * T * C;             // (B,C)
     const dim3 grid(B * H), block(256);
     {
-        const char* path = getenv("VRWKV_WKV6_BWD_PATH");            // "scalar" forces the sequential sweeps (testing)
-        if (!(path && path[0] == 's') && (long long)T * C < (1LL << 29)) {
+        if (!option(OPT_WKV6_BWD_SCALAR) && (long long)T * C < (1LL << 29)) {   // the option forces the sequential sweeps (testing)
             using namespace wkv6_detail;
             unsigned char* todo = reinterpret_cast<unsigned char*>(gu_part + (size_t)B * C);
             const dim3 blk(128);
+            hipLaunchKernelGGL(clear_flags_kernel, dim3((B * H + 255) / 256), dim3(256), 0, st, todo, B * H);
 #define VRWKV_SCAN(KIND, DIR, OUT) hipLaunchKernelGGL((wkv6_bwd_scan_kernel<IO, WT, KIND, DIR, EW>), grid, blk, 0, st, \
                                                       rr, kk, vv, ww, u, gy, OUT, a, gw, gu_part, todo, T, C, H)
             VRWKV_SCAN(SCAN_GR, 1, gr); VRWKV_SCAN(SCAN_GK, 1, gk); VRWKV_SCAN(SCAN_GV, 1, gv);

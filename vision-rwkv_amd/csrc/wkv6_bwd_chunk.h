@@ -26,7 +26,8 @@
 //
 // One 128-thread workgroup per (b,h) and pass; the descending pass is launched first and writes, the
 // ascending pass adds (old values fetched behind the matrix stage).  A sequence with a chunk that decays by
-// more than e^-60 is flagged in `todo` and left to the sequential kernels.
+// more than e^-60 is flagged in `todo` and left to the sequential kernels: the flags are cleared before the scans
+// and a scan only ever sets one, so a sequence that any of the six scans gave up on is redone.
 #pragma once
 #include "wkv6_fwd_chunk.h"
 
@@ -510,7 +511,6 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         gu_acc += __shfl_xor(gu_acc, 32);
         if (g == 0) gu_part[(size_t)b * C + h * HN + ocol] = gu_acc;
     }
-    if (threadIdx.x == 0) todo[bh] = 0;
 }
 
 }  // namespace wkv6_detail

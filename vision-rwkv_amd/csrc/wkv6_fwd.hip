@@ -69,10 +69,7 @@ int launch_chunked(const void* r, const void* k, const void* v, const void* w, c
     return check_launch("wkv6_fwd (chunked)");
 }
 
-bool force_scalar() {
-    const char* s = getenv("VRWKV_WKV6_PATH");           // tuning / testing override
-    return s && !strcmp(s, "scalar");
-}
+bool force_scalar() { return option(OPT_WKV6_FWD_SCALAR) != 0; }   // testing override
 
 template <typename IO, typename WT>
 int launch_any(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,

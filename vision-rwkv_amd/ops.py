@@ -266,14 +266,29 @@ def q_shift(input, shift_pixel=1, gamma=1 / 4, patch_resolution=None):
     B, N, C = input.shape
     x = input.transpose(1, 2).reshape(B, C, patch_resolution[0], patch_resolution[1])
     H, W = patch_resolution
-    g = int(C * gamma)
+    b1, b2, b3, b4 = _shift_bounds(C, gamma)
     out = torch.zeros_like(x)
-    out[:, 0:g, :, shift_pixel:W] = x[:, 0:g, :, 0:W - shift_pixel]
-    out[:, g:2 * g, :, 0:W - shift_pixel] = x[:, g:2 * g, :, shift_pixel:W]
-    out[:, 2 * g:3 * g, shift_pixel:H, :] = x[:, 2 * g:3 * g, 0:H - shift_pixel, :]
-    out[:, 3 * g:4 * g, 0:H - shift_pixel, :] = x[:, 3 * g:4 * g, shift_pixel:H, :]
-    out[:, 4 * g:, ...] = x[:, 4 * g:, ...]
+    out[:, 0:b1, :, shift_pixel:W] = x[:, 0:b1, :, 0:W - shift_pixel]
+    out[:, b1:b2, :, 0:W - shift_pixel] = x[:, b1:b2, :, shift_pixel:W]
+    out[:, b2:b3, shift_pixel:H, :] = x[:, b2:b3, 0:H - shift_pixel, :]
+    out[:, b3:b4, 0:H - shift_pixel, :] = x[:, b3:b4, shift_pixel:H, :]
+    out[:, b4:, ...] = x[:, b4:, ...]
     return out.flatten(2).transpose(1, 2)
+
+
+def _shift_bounds(C, gamma):
+    """Upper ends of the four shifted channel groups exactly as the reference cuts them (vrwkv.py:72-76):
+    int(C*gamma), int(C*gamma*2), int(C*gamma*3), int(C*gamma*4)."""
+    return int(C * gamma), int(C * gamma * 2), int(C * gamma * 3), int(C * gamma * 4)
+
+
+def _equal_quarters(C, gamma, head_dim):
+    """The kernels shift four groups of one width; true when the reference's cuts are of that kind (every
+    stock model: C a multiple of 4 with gamma = 1/4, or per-head quarters)."""
+    if head_dim:
+        return True
+    b = _shift_bounds(C, gamma)
+    return b == (b[0], 2 * b[0], 3 * b[0], 4 * b[0])
 
 
 def stack_mixes(mixes, device):
@@ -291,6 +306,11 @@ def q_shift_mix(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=None, hea
         raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
     B, T, C = x.shape
     Hp, Wp = patch_resolution
+    if not _equal_quarters(C, gamma, head_dim):
+        # unequal channel groups (C*gamma not an integer): the reference's slice copies, then the lerps
+        xx = q_shift(x, shift_pixel, gamma, patch_resolution)
+        tab = mix_table if mix_table is not None else stack_mixes(mixes, x.device)
+        return [(x.float() * m + xx.float() * (1 - m)).to(x.dtype) for m in tab]
     mix = mix_table if mix_table is not None else stack_mixes(mixes, x.device)
     if mix.shape != (len(mixes), C) or mix.dtype != torch.float32 or not mix.is_contiguous() or mix.device != x.device:
         raise RuntimeError("mix_table must be a contiguous float32 (n_mix, C) tensor on x's device")
@@ -596,4 +616,7 @@ def q_shift_mix_autograd(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=
         raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
     table = torch.stack([m.reshape(-1).float() for m in mixes])
     Hp, Wp = patch_resolution
+    if not _equal_quarters(x.shape[-1], gamma, head_dim):
+        xx = q_shift(x, shift_pixel, gamma, patch_resolution)
+        return [(x.float() * m + xx.float() * (1 - m)).to(x.dtype) for m in table]
     return list(_QShiftMix.apply(x, table, shift_pixel, gamma, Hp, Wp, head_dim))
