@@ -58,6 +58,17 @@ int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v
                     int B, int T, int C, int io_dtype,
                     void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* Bi-WKV forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as vrwkv_biwkv_fwd,
+ * but the long-sequence workspace is an array built into the library (4 MiB of device memory per GPU, held until the
+ * process ends) and the call allocates nothing.  Shapes whose workspace (vrwkv_biwkv_fwd_workspace_bytes) exceeds
+ * vrwkv_biwkv_fwd_static_max_workspace_bytes() are rejected with VRWKV_WORKSPACE_TOO_SMALL.  All calls on one GPU
+ * share that array: calls that may overlap on a GPU (different streams or threads) race; use vrwkv_biwkv_fwd with
+ * separate workspaces for those. */
+size_t vrwkv_biwkv_fwd_static_max_workspace_bytes(void);
+int vrwkv_biwkv_fwd_static(const float* w, const float* u, const void* k, const void* v, void* y,
+                           int B, int T, int C, int io_dtype, void* hip_stream);
+
 /* ---- Bi-WKV backward ------------------------------------------------------------------
  * Replaces bi_wkv_backward(w,u,k,v,gy) -> [gw,gu,gk,gv]
  *   (classification/mmcls_custom/models/backbones/cuda_new/bi_wkv.cpp:35-47, launcher

@@ -1,6 +1,8 @@
 // Entry points of the Bi-WKV forward (argument checks, plan, dtype dispatch); the kernels
 // are instantiated per element type in biwkv_fwd_{f32,bf16,f16}.hip.
 #include "biwkv_fwd_impl.h"
+#include <atomic>
+#include <mutex>
 
 namespace vrwkv {
 namespace biwkv_fwd_detail {
@@ -24,6 +26,43 @@ int validate(int B, int T, int C, int io_dtype) {
         set_error("biwkv_fwd: T*C must stay below 2^29 elements (got T=%d, C=%d)", T, C);
         return VRWKV_UNSUPPORTED_SHAPE;
     }
+    return VRWKV_OK;
+}
+
+// ---- workspace of the entry point that allocates nothing -------------------------------------------------------
+// The long-sequence path hands per-super-chunk aggregates from its first kernel to its second through a workspace
+// (B * nSC * 6 * C floats).  vrwkv_biwkv_fwd takes it from the caller; vrwkv_biwkv_fwd_static takes this array
+// instead, which every GPU the library runs on holds (at its own address) until the process ends.
+constexpr size_t kStaticWorkspaceBytes = 4u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device; looked up once per device (the array's name is a host-side
+// handle, not an address a kernel can use).
+int static_workspace(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("biwkv_fwd_static: cannot identify the current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return VRWKV_INVALID_ARG;
+    }
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p) {
+                set_error("biwkv_fwd_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+                return VRWKV_LAUNCH_FAILED;
+            }
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
     return VRWKV_OK;
 }
 
@@ -74,4 +113,23 @@ extern "C" int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, co
         case VRWKV_F16:  return biwkv_fwd_launch_io<__half>(p, w, u, k, v, y, ws, B, T, C, st);
     }
     return VRWKV_UNSUPPORTED_DTYPE;
+}
+
+extern "C" size_t vrwkv_biwkv_fwd_static_max_workspace_bytes(void) { return kStaticWorkspaceBytes; }
+
+extern "C" int vrwkv_biwkv_fwd_static(const float* w, const float* u, const void* k, const void* v, void* y,
+                                      int B, int T, int C, int io_dtype, void* hip_stream) {
+    int rc = validate(B, T, C, io_dtype);
+    if (rc != VRWKV_OK) return rc;
+    const size_t need = vrwkv_biwkv_fwd_workspace_bytes(B, T, C, io_dtype);
+    if (need > kStaticWorkspaceBytes) {
+        set_error("biwkv_fwd_static: B=%d, T=%d, C=%d needs a workspace of %zu bytes, the built-in one holds %zu; "
+                  "use vrwkv_biwkv_fwd with a caller-owned workspace", B, T, C, need, kStaticWorkspaceBytes);
+        return VRWKV_WORKSPACE_TOO_SMALL;
+    }
+    void* ws = nullptr;
+    rc = static_workspace(&ws);
+    if (rc != VRWKV_OK) return rc;
+    // every workspace entry the second kernel reads is written by the first one of the same call: nothing to clear
+    return vrwkv_biwkv_fwd(w, u, k, v, y, B, T, C, io_dtype, ws, kStaticWorkspaceBytes, hip_stream);
 }
