@@ -15,6 +15,8 @@ wkv6.py        bidirectional RWKV-6 scan in float64: sequential recurrence,
 qshift.py      q_shift / q_shift_multihead as explicit index loops.
 blocks.py      the element-wise block steps around the operators (row epilogues,
                VRWKV6 token mixes, GroupNorm x gate), row by row in float64.
+chunk_carry.py float64 model of the reference kernel's 32-way token split (what a
+               literal CUDA run would return; tests/test_reference_chunk_carry.py).
 torch_eager.py the same recurrences as PyTorch CPU-eager fp32 loops over T
                (what the benchmark times as its CPU baseline).
 c/             plain-C restatement of the recurrences (double accumulators),
