@@ -5,7 +5,7 @@ layer) at B=64, T=196, C=768, each on its own pre-generated seeded k, v (12 dist
 sets, 1.4 GB in fp32, so nothing stays cache-resident from call to call).  Inputs are resident
 in HBM before the timed region.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--io fp32|bf16] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--io fp32|bf16] [--no-cpu-baseline] [--no-sweep] ...
 """
 import argparse
 import math
@@ -19,8 +19,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes per launch of the fp32 kernel at this shape: rocprofv3 FETCH_SIZE + WRITE_SIZE of this
-# command with --calibrate-copy, each scaled by what it reads for that plain copy of known size.
+# command with --calibrate-copy, each scaled by what it reads for that plain copy of known size
+# (profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md holds the two counter runs and the arithmetic).
 MEASURED_TRAFFIC_FP32 = 115_874_000
+TRAFFIC_SOURCE = "profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md"
+REPEATS = 5                    # timed loops per figure; the median is reported
 LAYERS = 12
 B, T, C = 64, 196, 768
 
@@ -31,6 +34,63 @@ def baseline_wu(torch):
     w = (-5.0 + 8.0 * (c / (C - 1))) / T
     u = (math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / T
     return w.float(), u.float()
+
+
+def median_us(torch, fn, steps, warmup, calls_per_step=1, stream=None):
+    """Median over REPEATS timed loops of `steps` steps (HIP events on the stream the kernels run on), in
+    microseconds per call; also returns the per-loop values."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    reps = []
+    for _ in range(REPEATS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        reps.append(e0.elapsed_time(e1) * 1e3 / (steps * calls_per_step))
+    return sorted(reps)[len(reps) // 2], reps
+
+
+def error_report(y, ref):
+    """The two error measures of the parity tests, for one output against the float64 oracle."""
+    import numpy as np
+    y = np.asarray(y, np.float64)
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    d = np.abs(y - ref)
+    return {"metric": "max|y - ref| / max(|ref|, floor)", "max_abs_err": float(d.max()), "rms_ref": round(rms, 5),
+            "rel_err_floor_rms": float((d / np.maximum(np.abs(ref), rms)).max()),
+            "rel_err_floor_0.01rms": float((d / np.maximum(np.abs(ref), 1e-2 * rms)).max()),
+            "reference": "oracle/c (float64 two-pass recurrence) on the same inputs"}
+
+
+def config2_section(torch, ops, steps, warmup):
+    """Dense-prediction shape of the Mask R-CNN backbone: B=2, T=4150 (50 x 83 patches), C=768, bf16 I/O, fp32 state;
+    k, v ~ N(0,1) with 1 % of the tokens scaled x8 (all channels of a token).  One call per step."""
+    import numpy as np
+    from oracle import clib
+    Bn, Tn, Cn = 2, 4150, 768
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(2)
+    k = torch.randn(Bn, Tn, Cn, generator=g)
+    v = torch.randn(Bn, Tn, Cn, generator=g)
+    big = (torch.rand(Bn, Tn, 1, generator=g) < 0.01).float() * 7.0 + 1.0
+    k, v = (k * big).to(dev).bfloat16(), (v * big).to(dev).bfloat16()
+    c = torch.arange(Cn, dtype=torch.float64)
+    w = ((-5.0 + 8.0 * (c / (Cn - 1))) / Tn).float().to(dev)
+    u = ((math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / Tn).float().to(dev)
+    us, reps = median_us(torch, lambda: ops.bi_wkv_forward(w, u, k, v), steps, warmup)
+    y = ops.bi_wkv_forward(w, u, k, v)
+    ref = clib.biwkv_fwd(w.cpu().numpy(), u.cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy())
+    byt = 3 * Bn * Tn * Cn * 2 + 2 * Cn * 4
+    return {"workload": f"Bi-WKV forward B={Bn} T={Tn} C={Cn}, bf16 I/O, fp32 state, 1% of tokens x8, one call per step",
+            "us_per_call": round(us, 2), "repeats_us": [round(x, 2) for x in reps],
+            "roofline": {"bound": "hbm", "achieved": round(byt / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(byt / us / 1e3 / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": byt,
+                         "traffic": None},
+            "error": error_report(y.float().cpu().numpy(), ref)}
 
 
 def cpu_baseline(torch, n_calls):
@@ -68,25 +128,14 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
     r, k, v = (torch.randn(Bw, Tw, Cw, generator=g).to(dev).bfloat16() for _ in range(3))
     w = (torch.randn(Bw, Tw, Cw, generator=g) * 0.5 - 0.5).to(dev)
     u = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
-    for _ in range(warmup):
-        ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = []
-    for _ in range(5):                                             # median of five timed loops of `steps` calls
-        e0.record()
-        for _ in range(steps):
-            y = ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u)
-        e1.record()
-        torch.cuda.synchronize()
-        reps.append(e0.elapsed_time(e1) * 1e3 / steps)
-    us = sorted(reps)[len(reps) // 2]
+    us, reps = median_us(torch, lambda: ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u), steps, warmup)
     nchunk = (Tw + 31) // 32
     # per chunk, pass and value half (one wave): 36 MFMA 32x32x16 = 36 * 32768 flop
     mfma_flops = Bw * Hw * 2 * nchunk * 2 * 36 * 32768
     out = {
         "workload": f"wkv6 forward B={Bw} T={Tw} C={Cw} H={Hw}, bf16 r,k,v, fp32 w,y",
         "us_per_call": round(us, 2),
+        "repeats_us": [round(x, 2) for x in reps],
         "tokens_per_s": round(Bw * Tw / (us * 1e-6), 1),
         "recurrence_tflops": round(Bw * Tw * Hw * (10 * 64 * 64 + 3 * 64) / (us * 1e-6) / 1e12, 2),
         "mfma_issued_tflops": round(mfma_flops / (us * 1e-6) / 1e12, 2),
@@ -129,16 +178,7 @@ def backward_section(torch, ops, steps, warmup):
     u6 = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
 
     def timed(fn):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / steps
+        return median_us(torch, fn, steps, warmup)[0]
 
     us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
     us_6 = timed(lambda: ops.wkv6_backward(B, T, C, Hw, r6, k6, v6, w6, u6, gy))
@@ -164,16 +204,7 @@ def sweep_section(torch, ops, steps, warmup):
             u = ((math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / Tn).to(dev)
 
             def timed(fn):
-                for _ in range(warmup):
-                    fn()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(steps):
-                    fn()
-                e1.record()
-                torch.cuda.synchronize()
-                return e0.elapsed_time(e1) * 1e3 / steps
+                return median_us(torch, fn, steps, warmup)[0]
 
             us_f = timed(lambda: ops.bi_wkv_forward(w, u, k, v))
             us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
@@ -279,7 +310,8 @@ def main():
     ap.add_argument("--no-wkv6", action="store_true", help="skip the secondary wkv6 measurement")
     ap.add_argument("--no-backbone", action="store_true", help="skip the VRWKV-L whole-forward measurement")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-kernel measurements")
-    ap.add_argument("--sweep", action="store_true", help="also time Bi-WKV at the dense-prediction shapes (B=2, long T)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the dense-prediction shape sweep (B=2, long T)")
+    ap.add_argument("--no-config2", action="store_true", help="skip the B=2, T=4150, C=768 bf16 measurement")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -327,22 +359,11 @@ def main():
 
     if args.calibrate_copy:
         ys[0].float().copy_(ks[0].float()) if args.io != "fp32" else ys[0].copy_(ks[0])
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(args.steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    dev_ms = e0.elapsed_time(e1)
-    ms_per_step = max(dev_ms, 0.0) / args.steps
+    # W warm-up steps, then REPEATS timed loops of exactly K steps each (HIP events on the stream the kernels run
+    # on, device idle on both sides of every loop); the median loop is the reported one
+    us_per_launch, reps_us = median_us(torch, step, args.steps, args.warmup, LAYERS, stream)
+    ms_per_step = us_per_launch * LAYERS / 1e3
     n_launch = args.steps * LAYERS
-    us_per_launch = dev_ms * 1e3 / n_launch
     bytes_alg = 3 * B * T * C * esz + 2 * C * 4          # k, v read once, y written once, w and u
     gbs = bytes_alg / (us_per_launch * 1e-6) / 1e9
 
@@ -358,13 +379,15 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
+        "io_dtype": args.io,
         "data": "synthetic",
         "config": {"workload": f"Bi-WKV forward, VRWKV-B shape B={B} T={T} C={C}, {args.io} I/O, "
                                f"{LAYERS} back-to-back calls per step on distinct seeded k,v",
                    "io_dtype": args.io, "calls_per_step": LAYERS, "seed": 1234},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "us_per_call": round(us_per_launch, 3),
-        "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "timing": f"median of {REPEATS} loops of {args.steps} steps after {args.warmup} warm-up steps",
+        "repeats_us_per_call": [round(x, 3) for x in reps_us],
         "roofline": {
             "bound": "hbm",
             "achieved": round(gbs, 1),
@@ -372,6 +395,7 @@ def main():
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_FP32 if args.io == "fp32" else None,
+            "traffic_source": TRAFFIC_SOURCE if args.io == "fp32" else None,
             "kernel": "biwkv_fwd_kernel (one launch per call)",
             "algorithmic_bytes_per_launch": bytes_alg,
         },
@@ -389,29 +413,35 @@ def main():
                 if rc:
                     _lib.check(rc)
 
-        for _ in range(args.warmup):
-            step_h()
-        torch.cuda.synchronize()
-        h0, h1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        h0.record(stream)
-        for _ in range(args.steps):
-            step_h()
-        h1.record(stream)
-        torch.cuda.synchronize()
-        us_h = h0.elapsed_time(h1) * 1e3 / n_launch
+        us_h, reps_h = median_us(torch, step_h, args.steps, args.warmup, LAYERS, stream)
         bytes_h = 3 * B * T * C * 2 + 2 * C * 4
-        out["bf16_io"] = {"us_per_call": round(us_h, 3), "GBps": round(bytes_h / us_h / 1e3, 1),
-                          "pct_hbm_peak": round(100.0 * bytes_h / us_h / 1e3 / HBM_PEAK_GBS, 2),
-                          "algorithmic_bytes_per_launch": bytes_h}
+        out["bf16_io"] = {"us_per_call": round(us_h, 3), "repeats_us_per_call": [round(x, 3) for x in reps_h],
+                          "roofline": {"bound": "hbm", "achieved": round(bytes_h / us_h / 1e3, 1), "peak": HBM_PEAK_GBS,
+                                       "unit": "GB/s", "frac": round(bytes_h / us_h / 1e3 / HBM_PEAK_GBS, 4),
+                                       "traffic": None, "algorithmic_bytes_per_launch": bytes_h}}
+        if not args.no_cpu_baseline:
+            from oracle import clib
+            refh = clib.biwkv_fwd(w.cpu().numpy(), u.cpu().numpy(), kh[0].float().cpu().numpy(), vh[0].float().cpu().numpy())
+            out["bf16_io"]["error"] = error_report(yh[0].float().cpu().numpy(), refh)
         del kh, vh, yh
     if not args.no_cpu_baseline:
+        # layer 0's output against the float64 C oracle and against the CPU-eager fp32 recurrence the baseline times
+        # (both on the same k, v: the first two draws of seed 1234)
+        from oracle import clib
+        ref = clib.biwkv_fwd(w.cpu().numpy(), u.cpu().numpy(), ks[0].float().cpu().numpy(), vs[0].float().cpu().numpy())
+        out["error"] = error_report(ys[0].float().cpu().numpy(), ref)
+        out["error"]["tolerance"] = "1e-4 (fp32 I/O), 1e-2 (16-bit I/O) on the floor = rms(ref) measure (tests/conftest.py)"
         cb, y_cpu = cpu_baseline(torch, args.cpu_calls)
         out["cpu_baseline"] = cb
+        if args.io == "fp32":
+            out["error"]["cpu_eager_fp32_recurrence"] = error_report(y_cpu.numpy(), ref)["rel_err_floor_0.01rms"]
     if not args.no_wkv6:
         out["wkv6"] = wkv6_section(torch, ops, max(args.steps, 10), max(args.warmup // 5, 3), not args.no_cpu_baseline)
     if not args.no_backward:
         out["backward"] = backward_section(torch, ops, 10, 3)
-    if args.sweep:
+    if not args.no_config2:
+        out["config2"] = config2_section(torch, ops, 20, 10)
+    if not args.no_sweep:
         out["sweep"] = sweep_section(torch, ops, 10, 3)
     if not args.no_backbone:
         out["backbone"] = backbone_section(torch, ops, 5, 3)

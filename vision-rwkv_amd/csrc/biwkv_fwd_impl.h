@@ -130,8 +130,22 @@ struct BiwkvTile {
     // staging geometry: a lane moves 16 bytes = EPL elements; LPR lanes cover a 64-channel row; an instruction RPI rows
     static constexpr int EPL = 16 / (int)sizeof(IO), LPR = WAVE / EPL, RPI = WAVE / LPR;
     static constexpr int NI = (L + RPI - 1) / RPI, LR = NI * RPI;         // instructions and LDS rows per tensor
-    static constexpr bool OUT_STAGED = STAGED && sizeof(IO) == 2;         // 16-bit y goes out in 16-byte pieces as well
-    static constexpr int STAGE_ELEMS = (2 + (OUT_STAGED ? 1 : 0)) * LR * WAVE;   // per wave: k rows, v rows, (y rows)
+    // The wait for the next tile's rows stands before this tile's first store (loads and stores share one counter:
+    // a wait at the top of the next tile would also wait for the stores issued a moment before it).
+    static constexpr bool EARLY_WAIT = true;
+    // s_waitcnt vmcnt(0) as an instruction the compiler's own wait-count bookkeeping sees (it does not look into
+    // inline assembly and would add a wait of its own in front of the next read of a staged row)
+    static __device__ __forceinline__ void wait_vm0() {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt = 0, expcnt and lgkmcnt untouched
+        asm volatile("" ::: "memory");
+    }
+    // 16-bit y goes out in 16-byte pieces as well (through an LDS array of its own: an LDS read waits for every
+    // LDS-direct load that may write the array it reads).  fp32 y keeps its lane-per-channel 256-byte row stores:
+    // parked in LDS and flushed eight rows at a time it measured 2 % slower (24.6 vs 24.1 us at 64 x 196 x 768), the
+    // extra LDS round trip costing more than the wider stores save.
+    static constexpr bool OUT_STAGED = STAGED && sizeof(IO) == 2;
+    static constexpr int STAGE_ELEMS = 2 * LR * WAVE;                     // per wave: k rows, v rows
+    static constexpr int YSTAGE_ELEMS = OUT_STAGED ? LR * WAVE : 8;       // per wave: y rows
 
     const float* __restrict__ w_;
     const float* __restrict__ u_;
@@ -143,7 +157,8 @@ struct BiwkvTile {
     TileGeom g;
     int lane, wave, S;
     AggPtr s_agg0, s_agg1;      // two LDS exchange buffers, alternated tile by tile
-    IO* s_stage;                // STAGED: this wave's LDS rows [LR][64] of k, then v (then y for 16-bit I/O)
+    IO* s_stage;                // STAGED: this wave's LDS rows [LR][64] of k, then v
+    IO* s_y;                    // STAGED: this wave's LDS rows [YR][64] of y
 
     struct Where {
         int b, sc, ctile, c0, tw;
@@ -252,8 +267,9 @@ struct BiwkvTile {
             if (STAGED) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); else lds_barrier();
             if (next < g.n_tiles) {
                 if (STAGED) {
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the skipped tile's rows must have landed
+                    if (!EARLY_WAIT) wait_vm0();                          // the skipped tile's rows must have landed
                     issue_stage(next, wun);
+                    if (EARLY_WAIT) wait_vm0();                           // ... and the next tile's, before its turn
                 } else {
                     issue_loads(next, Kn, Vn, wun);
                 }
@@ -331,9 +347,10 @@ struct BiwkvTile {
         // unpack; tokens past T read as zero from the buffer and get k = -inf here
         float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
         if (STAGED) {
-            // this tile's rows have landed (loads and the previous tile's stores share one counter and may
-            // retire in either order, so the wait is for all of them)
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // This tile's rows have landed: the wait for them stands before the previous tile's first store (and
+            // before the loop for the first tile).  Loads and stores share one counter and may retire in either
+            // order, so a wait here would also wait for the stores that were issued a moment ago.
+            if (!EARLY_WAIT) wait_vm0();
             if (q.tw + L <= T) {                         // wave-uniform: every token of the chunk exists
 #pragma unroll
                 for (int j = 0; j < L; ++j) {
@@ -502,6 +519,7 @@ struct BiwkvTile {
 #pragma unroll
                 for (int j = 0; j < L; ++j) Vn[j].raw = load_raw(rvn, qn.voff0 + (unsigned)j * row);
             }
+            if (STAGED && EARLY_WAIT) wait_vm0();                         // the next tile's rows
             return;
         }
 
@@ -530,23 +548,33 @@ struct BiwkvTile {
                 c[e] = fmaf(gd[e], c[e], X1[j][e]);
                 d[e] = fmaf(gd[e], d[e], X0[j][e]);
             }
-            if (OUT_STAGED) s_stage[(2 * LR + j) * WAVE + lane] = from_f32<IO>(out[0]);
-            else buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
+            // the next tile's rows must have landed before this tile's first store joins them in the queue
+            if (STAGED && EARLY_WAIT && j == (OUT_STAGED ? 0 : L - 1)) wait_vm0();
+            if (OUT_STAGED) {
+                s_y[j * WAVE + lane] = from_f32<IO>(out[0]);
+                if (j == 0) flush_y(q, ry);
+            } else {
+                buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
+            }
         }
-        if (OUT_STAGED) {
-            // y rows of this wave, written lane-per-channel above, leave as 16-byte pieces (RPI rows per store)
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            const int cq = q.ctile * WAVE + (lane % LPR) * EPL;
+    }
+
+    // The y rows of this wave's chunk, parked lane-per-channel in the y region, leave as 16-byte pieces (RPI rows per
+    // store instruction); the region may be rewritten afterwards.
+    __device__ __forceinline__ void flush_y(const Where& q, __amdgpu_buffer_rsrc_t ry) const {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int cq = q.ctile * WAVE + (lane % LPR) * EPL;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < NI; ++i) {
+            {
                 const int rl = RPI * i + lane / LPR;
                 const int rowt = q.tw + rl;
                 const unsigned vo = (rl < L && rowt < T && cq < C) ? (unsigned)(((size_t)rowt * C + cq) * sizeof(IO)) : OOB_OFFSET;
-                const BufRaw<16>::type val = *reinterpret_cast<const BufRaw<16>::type*>(s_stage + (2 * LR + rl) * WAVE + (lane % LPR) * EPL);
+                const BufRaw<16>::type val = *reinterpret_cast<const BufRaw<16>::type*>(s_y + rl * WAVE + (lane % LPR) * EPL);
                 BufRaw<16>::template st<CPOL_NT>(val, ry, vo, 0);
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // the y rows are read before the next tile rewrites them
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                // the rows are read before they are rewritten
     }
 
     // Robust path of one tile, self-contained (own loads, no prefetch); a no-op for tiles the
@@ -694,6 +722,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     using Tile = BiwkvTile<IO, VEC, L, MODE, STAGED>;
     __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
     __shared__ __attribute__((aligned(16))) IO s_stage[STAGED ? Tile::SMAX : 1][STAGED ? Tile::STAGE_ELEMS : 1];
+    __shared__ __attribute__((aligned(16))) IO s_y[Tile::OUT_STAGED ? Tile::SMAX : 1][Tile::YSTAGE_ELEMS];
 
     Tile t;
     t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
@@ -704,6 +733,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     t.s_agg0 = s_agg[0];
     t.s_agg1 = s_agg[1];
     t.s_stage = &s_stage[STAGED ? t.wave : 0][0];
+    t.s_y = &s_y[Tile::OUT_STAGED ? t.wave : 0][0];
 
     typename Tile::P K0[L], V0[L], K1[L], V1[L];
     typename Tile::WU wu0, wu1;
@@ -714,6 +744,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     if ((gridDim.x & 7) == 0) tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     if (tile < g.n_tiles) {
         if (STAGED) t.issue_stage(tile, wu0); else t.issue_loads(tile, K0, V0, wu0);
+        if (STAGED && Tile::EARLY_WAIT) Tile::wait_vm0();                 // every tile starts with its rows landed
         for (;;) {
             int next = tile + gridDim.x;
             t.run(tile, next, 0, K0, V0, wu0, K1, V1, wu1);
