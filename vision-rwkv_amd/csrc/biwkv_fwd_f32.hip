@@ -5,3 +5,6 @@ namespace biwkv_fwd_detail {
 template int biwkv_fwd_launch_io<float>(const Plan&, const float*, const float*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
 }
 }
+#ifdef VRWKV_STAMPS
+VRWKV_DEFINE_STAMP_SETTER(f32)
+#endif

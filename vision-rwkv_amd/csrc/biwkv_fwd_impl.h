@@ -157,6 +157,7 @@ struct BiwkvTile {
     TileGeom g;
     int lane, wave, S;
     AggPtr s_agg0, s_agg1;      // two LDS exchange buffers, alternated tile by tile
+    float (*s_fold)[WAVE];      // MODE 2: [2][6][64] what the other super-chunks contribute, alternated like s_agg
     IO* s_stage;                // STAGED: this wave's LDS rows [LR][64] of k, then v
     IO* s_y;                    // STAGED: this wave's LDS rows [YR][64] of y
 
@@ -183,7 +184,20 @@ struct BiwkvTile {
 
     // Per-lane parameters of a tile, fetched together with its tokens so that consuming them
     // never has to wait for the previous tile's stores.
-    struct WU { float w[VEC], u[VEC]; };
+    // MODE 2 also fetches, together with a tile's parameters, the workspace entries of the other super-chunks of its
+    // sequence: wave 0 those of the earlier super-chunks (farthest first), wave 1 those of the later ones (farthest
+    // first), up to NBF each -- a whole tile ahead, so that folding them (fold_others) waits for no memory round trip.
+    static constexpr int NBF = MODE == 2 ? 16 : 1;
+    struct WU { float w[VEC], u[VEC]; float fr[NBF], f0[NBF], f1[NBF]; };
+
+    // super-chunk whose entry is the i-th one folded by `wave` (0: earlier ones ascending, 1: later ones descending)
+    __device__ __forceinline__ int fold_source(int i) const { return wave == 0 ? i : g.nSC - 1 - i; }
+    __device__ __forceinline__ float table_entry(const Where& q, int se, int slot) const {
+        // one descriptor over the batch element's table, the entry's offset in the scalar operand
+        const __amdgpu_buffer_rsrc_t rtab = make_rsrc(ws + (size_t)q.b * g.nSC * NSLOT * C, (unsigned)((size_t)g.nSC * NSLOT * C * 4));
+        const unsigned vcol = q.cok ? (unsigned)q.c0 * 4u : OOB_OFFSET;
+        return __builtin_bit_cast(float, BufRaw<4>::ld(rtab, vcol, (unsigned)((se * NSLOT + slot) * C) * 4u));
+    }
 
     __device__ __forceinline__ void issue_wu(int tile, WU& wu) const {
         const Where q = locate(tile);
@@ -192,6 +206,53 @@ struct BiwkvTile {
             wu.w[e] = q.cok ? w_[q.c0 + e] : 0.f;
             wu.u[e] = q.cok ? u_[q.c0 + e] : 0.f;
         }
+        if (MODE == 2 && wave < 2) {                     // wave-uniform
+#pragma unroll
+            for (int i = 0; i < NBF; ++i) {
+                int se = fold_source(i);                 // past the ends: clamped to an entry that exists, not used
+                se = se < 0 ? 0 : (se >= g.nSC ? g.nSC - 1 : se);
+                wu.fr[i] = table_entry(q, se, 2);
+                wu.f0[i] = table_entry(q, se, wave == 0 ? 0 : 3);
+                wu.f1[i] = table_entry(q, se, wave == 0 ? 1 : 4);
+            }
+        }
+    }
+
+    // MODE 2, waves 0 and 1: what the other super-chunks contribute to this tile -- wave 0: (A, B) of the earlier ones
+    // decayed to this super-chunk's first token; wave 1: (C, D) of the later ones decayed to its last -- left in LDS
+    // (s_fold[par]) for every wave to pick up after the tile's barrier.  The sum is kept at the running maximum of
+    // the scales met so far (all scales are integers, so re-scaling is an exact ldexp).
+    __device__ __forceinline__ void fold_others(const Where& q, const WU& wu, float om, int par) const {
+        auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
+        const int n = wave == 0 ? q.sc : g.nSC - 1 - q.sc;               // entries to fold
+        const float GS = fast_exp2(-om * (float)(S * L));
+        float r1 = NEG_BIG, aa = 0.f, ab = 0.f;
+        auto push = [&](float tr, float t0, float t1) {
+            const float m = fmaxf(r1, tr);
+            const int so = shift_of(r1, m), sn = shift_of(tr, m);
+            aa = fmaf(GS, ldexpf(aa, so), ldexpf(t0, sn));
+            ab = fmaf(GS, ldexpf(ab, so), ldexpf(t1, sn));
+            r1 = m;
+        };
+#pragma unroll
+        for (int i = 0; i < NBF; ++i)
+            if (i < n) push(wu.fr[i], wu.f0[i], wu.f1[i]);               // wave-uniform
+        for (int i0 = NBF; i0 < n; i0 += 8) {                            // longer sequences: the rest, eight at a time
+            float tr[8], t0[8], t1[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int se = fold_source(i0 + i);
+                se = se < 0 ? 0 : (se >= g.nSC ? g.nSC - 1 : se);
+                tr[i] = table_entry(q, se, 2);
+                t0[i] = table_entry(q, se, wave == 0 ? 0 : 3);
+                t1[i] = table_entry(q, se, wave == 0 ? 1 : 4);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i0 + i < n) push(tr[i], t0[i], t1[i]);
+        }
+        float (*f)[WAVE] = s_fold + (par * 6 + wave * 3);
+        f[0][lane] = r1; f[1][lane] = aa; f[2][lane] = ab;
     }
     static __device__ __forceinline__ typename BufRaw<sizeof(IO) * VEC>::type load_raw(__amdgpu_buffer_rsrc_t r, unsigned vo) {
         return BufRaw<sizeof(IO) * VEC>::template ld<CPOL_NT>(r, vo, 0);
@@ -260,6 +321,10 @@ struct BiwkvTile {
         const float NEG_INF = -__builtin_inff();
         const int nSC = g.nSC;
         const int li = lane * VEC;
+        const int round = tile / (int)gridDim.x + (MODE == 1 ? 2 : 0);   // which of this workgroup's tiles (cycle stamps;
+                                                                         // the aggregate-only pass uses slots 2, 3)
+        (void)round;
+        VRWKV_STAMP(wave, round, 0);                      // tile entered
 
         float om[VEC], mu[VEC];
         if (tile_is_robust(wu, om, mu)) {
@@ -293,57 +358,10 @@ struct BiwkvTile {
         if (have_next) issue_wu(next, wun);
 
         auto shift_of = [](float r_from, float r_to) -> int { return (int)fmaxf(r_from - r_to, -300.f); };
-        // MODE 2: what the other super-chunks contribute -- (A, B) of the earlier ones decayed to this super-chunk's first
-        // token, (C, D) of the later ones decayed to its last -- depends on the workspace alone and is folded here, before
-        // the tile's rows are touched.  Entries are fetched eight at a time (one memory round trip per batch instead of
-        // one per super-chunk); each direction keeps its sum at the running maximum of the scales met so far (all scales
-        // are integers, so re-scaling is an exact ldexp), and the two meet the tile's own scale after the exchange.
+        // MODE 2: what the other super-chunks contribute is folded by waves 0 and 1 from entries fetched a tile ago
         float ra[VEC], rc[VEC], ca[VEC], cb[VEC], cc[VEC], cd[VEC];
-        if (MODE == 2) {
-            constexpr int NB = 8;
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                float r1 = NEG_BIG, r2 = NEG_BIG, aa = 0.f, ab = 0.f, ac = 0.f, ad = 0.f;
-                if (q.cok) {
-                    const float GS = fast_exp2(-om[e] * (float)(S * L));
-                    for (int s0 = 0; s0 < q.sc; s0 += NB) {
-                        float tr[NB], t0[NB], t1[NB];
-#pragma unroll
-                        for (int i = 0; i < NB; ++i) {
-                            const int se = s0 + i;                                     // wave-uniform
-                            if (se < q.sc) { tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 0, e); t1[i] = ws_at(se, 1, e); }
-                        }
-#pragma unroll
-                        for (int i = 0; i < NB; ++i)
-                            if (s0 + i < q.sc) {
-                                const float m = fmaxf(r1, tr[i]);
-                                const int so = shift_of(r1, m), sn = shift_of(tr[i], m);
-                                aa = fmaf(GS, ldexpf(aa, so), ldexpf(t0[i], sn));
-                                ab = fmaf(GS, ldexpf(ab, so), ldexpf(t1[i], sn));
-                                r1 = m;
-                            }
-                    }
-                    for (int s0 = nSC - 1; s0 > q.sc; s0 -= NB) {
-                        float tr[NB], t0[NB], t1[NB];
-#pragma unroll
-                        for (int i = 0; i < NB; ++i) {
-                            const int se = s0 - i;
-                            if (se > q.sc) { tr[i] = ws_at(se, 2, e); t0[i] = ws_at(se, 3, e); t1[i] = ws_at(se, 4, e); }
-                        }
-#pragma unroll
-                        for (int i = 0; i < NB; ++i)
-                            if (s0 - i > q.sc) {
-                                const float m = fmaxf(r2, tr[i]);
-                                const int so = shift_of(r2, m), sn = shift_of(tr[i], m);
-                                ac = fmaf(GS, ldexpf(ac, so), ldexpf(t0[i], sn));
-                                ad = fmaf(GS, ldexpf(ad, so), ldexpf(t1[i], sn));
-                                r2 = m;
-                            }
-                    }
-                }
-                ra[e] = r1; rc[e] = r2; ca[e] = aa; cb[e] = ab; cc[e] = ac; cd[e] = ad;
-            }
-        }
+        if (MODE == 2 && wave < 2) fold_others(q, wu, om[0], par);
+        VRWKV_STAMP(wave, round, 1);                      // other super-chunks folded (MODE 2)
         // unpack; tokens past T read as zero from the buffer and get k = -inf here
         float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
         if (STAGED) {
@@ -367,7 +385,9 @@ struct BiwkvTile {
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
+            VRWKV_STAMP(wave, round, 2);                                  // rows copied from LDS
             if (next < g.n_tiles) issue_stage(next, wun);
+            VRWKV_STAMP(wave, round, 3);                                  // next tile's loads issued
         } else {
 #pragma unroll
             for (int j = 0; j < L; ++j) {
@@ -430,13 +450,21 @@ struct BiwkvTile {
             s_agg[wave][3][li + e] = Cg[e];
             s_agg[wave][4][li + e] = D[e];
         }
+        VRWKV_STAMP(wave, round, 4);                      // aggregate pass done, aggregates written
         if (STAGED) {
             // LDS-only barrier by hand: the fence form would also wait for the next tile's staging loads
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         } else {
             lds_barrier();
         }
+        VRWKV_STAMP(wave, round, 5);                      // barrier passed
 
+        if (MODE == 2) {
+            static_assert(MODE != 2 || VEC == 1, "the long-sequence emit pass handles one channel per lane");
+            const float (*f)[WAVE] = s_fold + par * 6;
+            ra[0] = f[0][lane]; ca[0] = f[1][lane]; cb[0] = f[2][lane];
+            rc[0] = f[3][lane]; cc[0] = f[4][lane]; cd[0] = f[5][lane];
+        }
         float G[VEC];                                     // decay over one wave's chunk
 #pragma unroll
         for (int e = 0; e < VEC; ++e) G[e] = fast_exp2(-om[e] * (float)L);
@@ -519,10 +547,13 @@ struct BiwkvTile {
 #pragma unroll
                 for (int j = 0; j < L; ++j) Vn[j].raw = load_raw(rvn, qn.voff0 + (unsigned)j * row);
             }
+            VRWKV_STAMP(wave, round, 8);
             if (STAGED && EARLY_WAIT) wait_vm0();                         // the next tile's rows
+            VRWKV_STAMP(wave, round, 9);
             return;
         }
 
+        VRWKV_STAMP(wave, round, 6);                      // carries formed
         // emit: ascending sweep leaves past + bonus partials, descending sweep adds the future
         float cu[VEC];
 #pragma unroll
@@ -539,6 +570,7 @@ struct BiwkvTile {
             }
             if (have_next) Vn[j].raw = load_raw(rvn, qn.voff0 + (unsigned)j * row);
         }
+        VRWKV_STAMP(wave, round, 7);                      // ascending sweep done
 #pragma unroll
         for (int j = L - 1; j >= 0; --j) {
             float out[VEC];
@@ -549,7 +581,11 @@ struct BiwkvTile {
                 d[e] = fmaf(gd[e], d[e], X0[j][e]);
             }
             // the next tile's rows must have landed before this tile's first store joins them in the queue
-            if (STAGED && EARLY_WAIT && j == (OUT_STAGED ? 0 : L - 1)) wait_vm0();
+            if (STAGED && EARLY_WAIT && j == (OUT_STAGED ? 0 : L - 1)) {
+                VRWKV_STAMP(wave, round, 8);              // (16-bit: descending sweep done) waiting for the next tile's rows
+                wait_vm0();
+                VRWKV_STAMP(wave, round, 9);              // next tile's rows have landed
+            }
             if (OUT_STAGED) {
                 s_y[j * WAVE + lane] = from_f32<IO>(out[0]);
                 if (j == 0) flush_y(q, ry);
@@ -557,6 +593,7 @@ struct BiwkvTile {
                 buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);   // tokens >= T fall outside the descriptor
             }
         }
+        VRWKV_STAMP(wave, round, 10);                     // descending sweep done, stores issued
     }
 
     // The y rows of this wave's chunk, parked lane-per-channel in the y region, leave as 16-byte pieces (RPI rows per
@@ -723,6 +760,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
     __shared__ __attribute__((aligned(16))) IO s_stage[STAGED ? Tile::SMAX : 1][STAGED ? Tile::STAGE_ELEMS : 1];
     __shared__ __attribute__((aligned(16))) IO s_y[Tile::OUT_STAGED ? Tile::SMAX : 1][Tile::YSTAGE_ELEMS];
+    __shared__ float s_fold[MODE == 2 ? 12 : 1][WAVE];
 
     Tile t;
     t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
@@ -732,6 +770,7 @@ void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_
     t.S = blockDim.x >> 6;
     t.s_agg0 = s_agg[0];
     t.s_agg1 = s_agg[1];
+    t.s_fold = s_fold;
     t.s_stage = &s_stage[STAGED ? t.wave : 0][0];
     t.s_y = &s_y[Tile::OUT_STAGED ? t.wave : 0][0];
 
@@ -812,7 +851,7 @@ inline Plan make_plan(int B, int T, int C, int io_dtype) {
         p.L = 28;
         for (int i = 0; i < kNumL; ++i) if (el == kLs[i]) p.L = el;
         p.S = smax_for(p.L, p.VEC);
-        if (es >= 1 && es <= smax_for(p.L, p.VEC)) p.S = es;
+        if (es >= 2 && es <= smax_for(p.L, p.VEC)) p.S = es;      // at least two waves: the emit pass gives two of them a job of their own
         p.nSC = (T + p.S * p.L - 1) / (p.S * p.L);
     }
     const int cap = smax_for(p.L, p.VEC);

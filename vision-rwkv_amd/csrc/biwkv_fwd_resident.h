@@ -119,13 +119,13 @@ __device__ __forceinline__ void resident_robust(const float* w_, const float* u_
     const int S = blockDim.x >> 6;
     BiwkvTile<IO, 1, L, 1, false> t1;
     t1.w_ = w_; t1.u_ = u_; t1.k_ = k_; t1.v_ = v_; t1.y_ = y_; t1.ws = ws; t1.T = T; t1.C = C; t1.g = g;
-    t1.lane = lane; t1.wave = wave; t1.S = S; t1.s_agg0 = agg0; t1.s_agg1 = agg1; t1.s_stage = nullptr; t1.s_y = nullptr;
+    t1.lane = lane; t1.wave = wave; t1.S = S; t1.s_agg0 = agg0; t1.s_agg1 = agg1; t1.s_stage = nullptr; t1.s_y = nullptr; t1.s_fold = nullptr;
     for (int sc = 0; sc < NSC; ++sc) t1.run_robust((b * NSC + sc) * n_ctile + ctile);
     __threadfence();
     __syncthreads();
     BiwkvTile<IO, 1, L, 2, false> t2;
     t2.w_ = w_; t2.u_ = u_; t2.k_ = k_; t2.v_ = v_; t2.y_ = y_; t2.ws = ws; t2.T = T; t2.C = C; t2.g = g;
-    t2.lane = lane; t2.wave = wave; t2.S = S; t2.s_agg0 = agg0; t2.s_agg1 = agg1; t2.s_stage = nullptr; t2.s_y = nullptr;
+    t2.lane = lane; t2.wave = wave; t2.S = S; t2.s_agg0 = agg0; t2.s_agg1 = agg1; t2.s_stage = nullptr; t2.s_y = nullptr; t2.s_fold = nullptr;
     for (int sc = 0; sc < NSC; ++sc) t2.run_robust((b * NSC + sc) * n_ctile + ctile);
 }
 

@@ -106,6 +106,30 @@ template <> struct BufRaw<16> {
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
+// ---- per-phase cycle stamps (instrumented build only: -DVRWKV_STAMPS, `make stamps`) ----------------------------
+// A wave records the shader clock at numbered points of a tile into a buffer the host registered with
+// vrwkv_debug_set_stamp_buffer: layout [workgroup][wave (8)][tile slot (VRWKV_STAMP_TILES)][point (VRWKV_STAMP_POINTS)].
+#ifdef VRWKV_STAMPS
+constexpr int VRWKV_STAMP_TILES = 4, VRWKV_STAMP_POINTS = 12;
+static __device__ unsigned long long* g_stamp_buffer = nullptr;   // one per translation unit (device code is not linked across them)
+// defines vrwkv_debug_set_stamp_buffer_<tag>(device_buffer) for the translation unit it is used in
+#define VRWKV_DEFINE_STAMP_SETTER(tag)                                                                      \
+    extern "C" int vrwkv_debug_set_stamp_buffer_##tag(void* device_buffer) {                                 \
+        unsigned long long* p = static_cast<unsigned long long*>(device_buffer);                             \
+        return hipMemcpyToSymbol(HIP_SYMBOL(::vrwkv::g_stamp_buffer), &p, sizeof(p)) == hipSuccess ? 0 : 4;   \
+    }
+__device__ __forceinline__ void stamp(int wave, int slot, int point) {
+    unsigned long long* buf = g_stamp_buffer;
+    if (buf && slot < VRWKV_STAMP_TILES && (threadIdx.x & 63) == 0) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        buf[(((size_t)blockIdx.x * 8 + wave) * VRWKV_STAMP_TILES + slot) * VRWKV_STAMP_POINTS + point] = __builtin_amdgcn_s_memtime();
+    }
+}
+#define VRWKV_STAMP(wave, slot, point) ::vrwkv::stamp(wave, slot, point)
+#else
+#define VRWKV_STAMP(wave, slot, point) ((void)0)
+#endif
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
