@@ -25,7 +25,7 @@
 // bf16 ones are exact.
 //
 // One 128-thread workgroup per (b,h) and pass; the descending pass is launched first and writes, the
-// ascending pass adds (old values fetched behind the matrix stage).  A sequence with a chunk that decays by
+// ascending pass adds (no-return atomics, put_f32).  A sequence with a chunk that decays by
 // more than e^-60 is flagged in `todo` and left to the sequential kernels: the flags are cleared before the scans
 // and a scan only ever sets one, so a sequence that any of the six scans gave up on is redone.
 #pragma once
@@ -35,6 +35,19 @@ namespace vrwkv {
 namespace wkv6_detail {
 
 enum { SCAN_GR = 0, SCAN_GK = 1, SCAN_GV = 2 };
+
+// One fp32 result of a scan: the descending pass (launched first) stores it, the ascending pass adds its own with a
+// no-return atomic at the L2 (every address is touched once per pass, so the sum does not depend on any order) --
+// no old values to fetch and to keep in registers.  Rows past T fall to the descriptor's range check either way.
+template <bool ADD>
+__device__ __forceinline__ void put_f32(float val, __amdgpu_buffer_rsrc_t r, unsigned voff) {
+    if (ADD) (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, r, voff, 0, 0);
+    else {
+        unsigned bits;
+        __builtin_memcpy(&bits, &val, 4);
+        BufRaw<4>::st(bits, r, voff, 0);
+    }
+}
 
 template <bool QS, bool KS>
 struct __attribute__((aligned(16))) ScanLds {
@@ -276,13 +289,11 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
 
         // ================================= stage M: matrix cores ===============================
         // values the epilogue needs in the output layout (lane = column ocol, register r = scan row)
-        float prev[16];
         RawIO rraw[16], kraw[16];
-        unsigned araw[16], pgw[16];
+        unsigned araw[16];
         RawW wo[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            if (KIND != SCAN_GK) prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
             if (KIND != SCAN_GV) {
                 rraw[r] = BufRaw<ES>::ld(rsr, row_off(cc, r, Cs, ES), 0);
                 kraw[r] = BufRaw<ES>::ld(rsk, row_off(cc, r, Cs, ES), 0);
@@ -410,8 +421,6 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             for (int r = 0; r < 16; ++r) {
                 araw[r] = BufRaw<4>::ld(rsa, row_off(cc, r, Cs, 4), 0);
                 wo[r] = BufRaw<sizeof(WT)>::ld(rsw, row_off(cc, r, Cs, sizeof(WT)), 0);
-                prev[r] = ASC ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
-                pgw[r] = ASC ? BufRaw<4>::ld(rsgw, row_off(cc, r, Cs, 4), 0) : 0u;
             }
         }
         // ---- MFMA 4: M[c][o] = sum_s Kc[s][c] Val[s][o];  state' = decay * state + scale * M ----
@@ -448,7 +457,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         if (KIND == SCAN_GV) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rso, row_off(cc, r, Cs, 4), 0);
+                put_f32<ASC>(accY[r], rso, row_off(cc, r, Cs, 4));
         } else {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");       // Diag: written and read inside a wave
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -465,12 +474,12 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     const float px = post * accY[r];
                     if (KIND == SCAN_GR) {
                         const float gr = fmaf(u_o * kk, dg[e], px);
-                        BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + gr), rso, row_off(cc, r, Cs, 4), 0);
+                        put_f32<ASC>(gr, rso, row_off(cc, r, Cs, 4));
                         BufRaw<4>::st(__builtin_bit_cast(unsigned, rr * px), rsa, row_off(cc, r, Cs, 4), 0);
                         gu_acc = fmaf(rr * kk, dg[e], gu_acc);
                     } else {
                         const float gk = fmaf(u_o * rr, dg[e], px);
-                        BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + gk), rso, row_off(cc, r, Cs, 4), 0);
+                        put_f32<ASC>(gk, rso, row_off(cc, r, Cs, 4));
                         dd[r] = __builtin_bit_cast(float, araw[r]) - kk * px;     // rows past T: a = 0, k = 0
                     }
                 }
@@ -496,8 +505,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                         const float fw = cvtw(wo[r]);
                         const float ldn = W_IS_EW ? fw : -__expf(fw);
                         const float gw = ldn * (run - bn);
-                        BufRaw<4>::st(__builtin_bit_cast(unsigned, __builtin_bit_cast(float, pgw[r]) + gw), rsgw,
-                                      row_off(cc, r, Cs, 4), 0);
+                        put_f32<ASC>(gw, rsgw, row_off(cc, r, Cs, 4));
                         run += dd[r];
                     }
                     before += bs[r4] + pbs[r4];
