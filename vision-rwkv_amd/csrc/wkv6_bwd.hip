@@ -242,11 +242,6 @@ void wkv6_bwd_fallback(const IO* r_, const IO* k_, const IO* v_, const WT* w_, c
     wkv6_bwd_sweep_v_body<IO, WT, 0, W_IS_EW>(bh, r_, k_, w_, u_, gy_, gv_, T, C, H);
 }
 
-__global__ void clear_flags_kernel(unsigned char* flags, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) flags[i] = 0;
-}
-
 template <typename IO, typename WT, bool EW>
 int launch_all(const void* r, const void* k, const void* v, const void* w, const float* u, const float* gy,
                float* gr, float* gk, float* gv, float* gw, float* gu, float* ws, int B, int T, int C, int H, hipStream_t st) {
@@ -262,9 +257,9 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
             using namespace wkv6_detail;
             unsigned char* todo = reinterpret_cast<unsigned char*>(gu_part + (size_t)B * C);
             const dim3 blk(128);
-            hipLaunchKernelGGL(clear_flags_kernel, dim3((B * H + 255) / 256), dim3(256), 0, st, todo, B * H);
 #define VRWKV_SCAN(KIND, DIR, OUT) hipLaunchKernelGGL((wkv6_bwd_scan_kernel<IO, WT, KIND, DIR, EW>), grid, blk, 0, st, \
                                                       rr, kk, vv, ww, u, gy, OUT, a, gw, gu_part, todo, T, C, H)
+            // gr descending first: it clears the fallback flags
             VRWKV_SCAN(SCAN_GR, 1, gr); VRWKV_SCAN(SCAN_GK, 1, gk); VRWKV_SCAN(SCAN_GV, 1, gv);
             VRWKV_SCAN(SCAN_GR, 0, gr); VRWKV_SCAN(SCAN_GK, 0, gk); VRWKV_SCAN(SCAN_GV, 0, gv);
 #undef VRWKV_SCAN

@@ -21,10 +21,9 @@
 // that same order); likewise A goes from the accumulators of MFMA 1 into the A operand of MFMA 2.
 //
 // y: both passes walk the same chunk grid from opposite ends.  The pass that reaches a chunk at the
-// earlier step stores, the other one adds at its (later) step with a no-return atomic at the L2, after the
-// barrier that ends every step (at the middle chunk of an odd count the descending pass stores before that
-// barrier and the ascending pass adds after it) -- y is never zero-filled or read back, and there is no
-// second launch.  Every y is the sum of exactly two terms, so the order of the two passes leaves no trace.
+// earlier step stores, the other one adds at its (later) step, after the barrier that ends every step (at
+// the middle chunk of an odd count the descending pass stores before that barrier and the ascending pass
+// adds after it) -- y is never zero-filled, and there is no second launch.
 //
 // Precision: every operand that is computed rather than loaded (rt, kt, A, S) is split into a
 // bf16 head and a bf16 tail and the products head*head + head*tail + tail*head are accumulated,
@@ -307,9 +306,16 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // ================================= stage M: matrix cores ===============================
         const int icol = 32 * q + x;                                      // value column of this lane
         // y: the other pass reaches this chunk at step nchunk-1-ch.  If that was earlier, its values are in
-        // memory already (made visible by that step's closing barrier) and this pass adds to them.
+        // memory already (made visible by that step's closing barrier): fetch them now, behind the MFMAs.
         const int cy = chunk_of(ch);
         const bool y_second = ch > nchunk - 1 - ch, y_tie = asc && ch == nchunk - 1 - ch;     // wave-uniform
+        float prev[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) prev[r] = 0.f;
+        if (y_second) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r, Cs), 0));
+        }
         // ---- MFMA 1: A^T: acc[m = s][n = t]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
         f32x16 accA = {0};
 #pragma unroll
@@ -410,32 +416,21 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // ---- y: store (sum with the other pass's value where it came first); on a tie the descending pass
         //      stores here and the ascending pass adds after the barrier ----
         if (!y_tie) {
-            if (y_second) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(accY[r], rsy, y_off(cy, r, Cs), 0, 0);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    // (as a scalar float first: a bit cast applied to the vector element itself has been seen to
-                    // store element 0 in every row)
-                    const float val = accY[r];
-                    unsigned bits;
-                    __builtin_memcpy(&bits, &val, 4);
-                    BufRaw<4>::st(bits, rsy, y_off(cy, r, Cs), 0);
-                }
-            }
+            for (int r = 0; r < 16; ++r)
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r, Cs), 0);
         }
         // end of the step: every LDS read of this chunk is done, and the stores above become visible
-        // to the other pass of this workgroup.  At the middle chunk of an odd count the other pass adds to these very
-        // rows right after the barrier: there the stores must have been performed (at the L2, where the adds
-        // happen) before the barrier is passed; everywhere else a whole step lies in between.
-        if (!asc && ch == nchunk - 1 - ch) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
+        // to the other pass of this workgroup
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();                                    // (3)
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (y_tie) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(accY[r], rsy, y_off(cy, r, Cs), 0, 0);
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rsy, y_off(cy, r, Cs), 0));
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                BufRaw<4>::st(__builtin_bit_cast(unsigned, prev[r] + accY[r]), rsy, y_off(cy, r, Cs), 0);
         }
     }
 
