@@ -18,11 +18,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-# HBM bytes per launch of the fp32 kernel at this shape: rocprofv3 FETCH_SIZE + WRITE_SIZE of this
+# HBM bytes per launch of the kernel at this shape: rocprofv3 FETCH_SIZE + WRITE_SIZE of this
 # command with --calibrate-copy, each scaled by what it reads for that plain copy of known size
-# (profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md holds the two counter runs and the arithmetic).
-MEASURED_TRAFFIC_FP32 = 115_874_000
-TRAFFIC_SOURCE = "profiles/biwkv_fwd_vrwkvB_fp32_hbm_traffic.md"
+# (profiles/biwkv_fwd_vrwkvB_hbm_traffic.md holds the two counter runs and the arithmetic).
+MEASURED_TRAFFIC_FP32 = 115_947_000
+MEASURED_TRAFFIC_BF16 = 58_172_000
+TRAFFIC_SOURCE = "profiles/biwkv_fwd_vrwkvB_hbm_traffic.md"
 REPEATS = 5                    # timed loops per figure; the median is reported
 LAYERS = 12
 B, T, C = 64, 196, 768
@@ -394,8 +395,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_FP32 if args.io == "fp32" else None,
-            "traffic_source": TRAFFIC_SOURCE if args.io == "fp32" else None,
+            "traffic": MEASURED_TRAFFIC_FP32 if args.io == "fp32" else MEASURED_TRAFFIC_BF16 if args.io == "bf16" else None,
+            "traffic_source": TRAFFIC_SOURCE if args.io in ("fp32", "bf16") else None,
             "kernel": "biwkv_fwd_kernel (one launch per call)",
             "algorithmic_bytes_per_launch": bytes_alg,
         },
@@ -418,7 +419,8 @@ def main():
         out["bf16_io"] = {"us_per_call": round(us_h, 3), "repeats_us_per_call": [round(x, 3) for x in reps_h],
                           "roofline": {"bound": "hbm", "achieved": round(bytes_h / us_h / 1e3, 1), "peak": HBM_PEAK_GBS,
                                        "unit": "GB/s", "frac": round(bytes_h / us_h / 1e3 / HBM_PEAK_GBS, 4),
-                                       "traffic": None, "algorithmic_bytes_per_launch": bytes_h}}
+                                       "traffic": MEASURED_TRAFFIC_BF16, "traffic_source": TRAFFIC_SOURCE,
+                                       "algorithmic_bytes_per_launch": bytes_h}}
         if not args.no_cpu_baseline:
             from oracle import clib
             refh = clib.biwkv_fwd(w.cpu().numpy(), u.cpu().numpy(), kh[0].float().cpu().numpy(), vh[0].float().cpu().numpy())
