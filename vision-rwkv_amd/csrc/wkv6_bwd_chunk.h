@@ -25,7 +25,7 @@
 // bf16 ones are exact.
 //
 // One 128-thread workgroup per (b,h) and pass; the descending pass is launched first and writes, the
-// ascending pass adds (no-return atomics, put_f32).  A sequence with a chunk that decays by
+// ascending pass adds (put_f32).  A sequence with a chunk that decays by
 // more than e^-60 is flagged in `todo` and left to the sequential kernels: the first scan launched (gr, descending)
 // clears its sequence's flag on entry and a scan only ever sets one, so a sequence that any of the six scans gave
 // up on is redone.
@@ -37,11 +37,13 @@ namespace wkv6_detail {
 
 enum { SCAN_GR = 0, SCAN_GK = 1, SCAN_GV = 2 };
 
+
 // One fp32 result of a scan: the descending pass (launched first) stores it, the ascending pass adds its own.  The
-// gk / gw scan, which has no registers left for the old values, adds with a no-return atomic at the L2 (every address
-// is touched once per pass, so the sum does not depend on any order); the gr and gv scans fetch the old values behind
-// their matrix stage and store the sums (4 us per scan faster than the atomics at 64 x 196 x 768).  Rows past T fall
-// to the descriptor's range check either way.
+// gr and gv scans fetch the old values behind their matrix stage and store the sums; the gk / gw scan has no registers
+// left for that: it fetches the old gk rows just before its epilogue and adds gw with a no-return atomic at the L2
+// (every address is touched once per pass, so the sum does not depend on any order).  Measured at 64 x 196 x 768: an
+// atomic costs about 1.2 us per million, a read-modify-write whose loads are hidden about a quarter of that.  Rows past
+// T fall to the descriptor's range check either way.
 template <bool ADD>
 __device__ __forceinline__ void put_f32(float val, __amdgpu_buffer_rsrc_t r, unsigned voff) {
     if (ADD) (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, r, voff, 0, 0);
@@ -52,13 +54,14 @@ __device__ __forceinline__ void put_f32(float val, __amdgpu_buffer_rsrc_t r, uns
     }
 }
 
-template <bool QS, bool KS>
+template <bool QS, bool KS, bool GW>
 struct __attribute__((aligned(16))) ScanLds {
     __bf16 Qh[LC][PJ], Ql[QS ? LC : 1][PJ];               // Q rows   [rho][c]
     __bf16 Kh[LC][PJ], Kl[KS ? LC : 1][PJ];               // Kc rows  [rho][c]
     __bf16 KTh[HN][PS], KTl[KS ? HN : 1][PS];             // Kc^T     [c][rho]
     __bf16 VTh[HN][PS], VTl[HN][PS];                      // Val^T    [o][rho]
     float Post[LC][HN];                                   // f1 / f2 in [rho][j]  (GR, GK)
+    float Ld[GW ? LC : 1][HN];                            // -log2 of the decay in [rho][j]  (GK: the factor of gw)
     float C1[HN], C2[HN], C3[HN], Tot[HN], Bon[4][LC], Diag[LC];
 };
 
@@ -82,7 +85,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     constexpr bool KS = KIND != SCAN_GR || !EXACT;         // Kc is computed (gy, rt) -> split; bf16 v is exact
     constexpr bool ASC = DIR == 0;
     constexpr bool LL = KIND != SCAN_GV;                   // tail x tail products too: gw is a difference of these sums
-    __shared__ ScanLds<QS, KS> L;
+    __shared__ ScanLds<QS, KS, KIND == SCAN_GK> L;
     __shared__ int sFlag;
 
     const int lane = threadIdx.x & 63;
@@ -198,6 +201,10 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 for (int m = 0; m < 16; ++m)
                     if (token_of_n(cc, 16 * q + m) >= T) e[m] = 0.f;
             }
+            if (KIND == SCAN_GK) {                                        // scan row of pass index 16q + m: 16(1-q) + 15 - m
+#pragma unroll
+                for (int m = 0; m < 16; ++m) L.Ld[16 * (1 - q) + 15 - m][lane] = e[m];
+            }
             p[0] = -e[0];
 #pragma unroll
             for (int m = 1; m < 16; ++m) p[m] = p[m - 1] - e[m];
@@ -297,17 +304,18 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // ================================= stage M: matrix cores ===============================
         // values the epilogue needs in the output layout (lane = column ocol, register r = scan row)
         constexpr bool RMW = ASC && KIND != SCAN_GK;      // ascending gr / gv: old values fetched here, sums stored
+        constexpr bool GK_RMW = ASC && KIND == SCAN_GK;   // ascending gk: old values fetched just before the epilogue
         float prev[16];
         RawIO rraw[16], kraw[16];
         unsigned araw[16];
-        RawW wo[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             prev[r] = RMW ? __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0)) : 0.f;
-            if (KIND != SCAN_GV) {
-                rraw[r] = BufRaw<ES>::ld(rsr, row_off(cc, r, Cs, ES), 0);
-                kraw[r] = BufRaw<ES>::ld(rsk, row_off(cc, r, Cs, ES), 0);
-            }
+            // the bonus terms (u k for gr, u r for gk) exist in the ascending pass only
+            if (KIND == SCAN_GR || (KIND == SCAN_GK && ASC)) rraw[r] = BufRaw<ES>::ld(rsr, row_off(cc, r, Cs, ES), 0);
+            else rraw[r] = RawIO{};
+            if (KIND == SCAN_GK || (KIND == SCAN_GR && ASC)) kraw[r] = BufRaw<ES>::ld(rsk, row_off(cc, r, Cs, ES), 0);
+            else kraw[r] = RawIO{};
         }
         // ---- MFMA 1: A^T: acc[s][t] = sum_c Kc[s][c] Q[t][c]; lane holds t = x, rows s = 8(r/4)+4g+(r%4) ----
         f32x16 accA = {0};
@@ -430,7 +438,6 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 araw[r] = BufRaw<4>::ld(rsa, row_off(cc, r, Cs, 4), 0);
-                wo[r] = BufRaw<sizeof(WT)>::ld(rsw, row_off(cc, r, Cs, sizeof(WT)), 0);
             }
         }
         // ---- MFMA 4: M[c][o] = sum_s Kc[s][c] Val[s][o];  state' = decay * state + scale * M ----
@@ -464,6 +471,10 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             }
         }
         // ================================== epilogue ==================================
+        if (GK_RMW) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) prev[r] = __builtin_bit_cast(float, BufRaw<4>::ld(rso, row_off(cc, r, Cs, 4), 0));
+        }
         if (KIND == SCAN_GV) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -483,13 +494,13 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     const float rr = cvt(rraw[r]), kk = cvt(kraw[r]);
                     const float px = post * accY[r];
                     if (KIND == SCAN_GR) {
-                        const float gr = fmaf(u_o * kk, dg[e], px);
+                        const float gr = ASC ? fmaf(u_o * kk, dg[e], px) : px;
                         put_f32<false>(prev[r] + gr, rso, row_off(cc, r, Cs, 4));
                         BufRaw<4>::st(__builtin_bit_cast(unsigned, rr * px), rsa, row_off(cc, r, Cs, 4), 0);
-                        gu_acc = fmaf(rr * kk, dg[e], gu_acc);
+                        if (ASC) gu_acc = fmaf(rr * kk, dg[e], gu_acc);
                     } else {
-                        const float gk = fmaf(u_o * rr, dg[e], px);
-                        put_f32<ASC>(gk, rso, row_off(cc, r, Cs, 4));
+                        const float gk = ASC ? fmaf(u_o * rr, dg[e], px) : px;
+                        put_f32<false>(prev[r] + gk, rso, row_off(cc, r, Cs, 4));
                         dd[r] = __builtin_bit_cast(float, araw[r]) - kk * px;     // rows past T: a = 0, k = 0
                     }
                 }
@@ -512,8 +523,7 @@ void wkv6_bwd_scan_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                         const int r = 4 * r4 + e;
                         const float kk = cvt(kraw[r]);
                         const float bn = kk * L.Post[8 * r4 + 4 * g + e][ocol] * accY[r];
-                        const float fw = cvtw(wo[r]);
-                        const float ldn = W_IS_EW ? fw : -__expf(fw);
+                        const float ldn = -L.Ld[8 * r4 + 4 * g + e][ocol] * (1.0f / LOG2E);   // log decay of the row's token
                         const float gw = ldn * (run - bn);
                         put_f32<ASC>(gw, rsgw, row_off(cc, r, Cs, 4));
                         run += dd[r];
