@@ -137,7 +137,7 @@ int launch(const float* w, const float* u, const void* k, const void* v, const v
             hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,
                                kk, vv, gg, ok, ov, ws, gw_part, gu_part, B, T, C);
     }
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gw_part, gw, gu_part, gu, B * p.nSC, C);
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, gw_part, gw, gu_part, gu, B * p.nSC, C);
     return check_launch("biwkv_bwd");
 }
 

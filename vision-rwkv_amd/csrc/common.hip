@@ -50,6 +50,13 @@ int option(Option o) {
     return g_options[o].load(std::memory_order_relaxed);
 }
 
+int device_cus() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    return n;
+}
+
 int check_launch(const char* what) {
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess) return VRWKV_OK;

@@ -317,7 +317,7 @@ int launch_gn_bwd(const void* y, const void* gate, const void* w, const void* b,
     }
 #undef VRWKV_GNB
     const int wide = 2 * C;                                   // gparam: (2, C) = g_weight, g_bias
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gparam, (const float*)nullptr,
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, part, gparam, (const float*)nullptr,
                        (float*)nullptr, (int)nblk, wide);
     return check_launch("groupnorm_gate_bwd");
 }
@@ -438,7 +438,7 @@ extern "C" int vrwkv_maa_mix_bwd(const void* x, const void* sx, const void* m, c
     }
 #undef VRWKV_MAAB
     const int wide = 5 * C;
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gmaa, (const float*)nullptr,
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, part, gmaa, (const float*)nullptr,
                        (float*)nullptr, (int)nrb, wide);
     return check_launch("maa_mix_bwd");
 }

@@ -20,48 +20,67 @@
 namespace vrwkv {
 namespace {
 
+constexpr int QF_CX = 32, QF_TY = 8;   // forward workgroup: 32 channel vectors x 8 token lanes
+constexpr int QF_TPT = 4;              // tokens per thread: a workgroup covers up to 32 tokens of 32 channel vectors
+
+// A thread keeps one channel vector's mix values in registers and walks QF_TPT tokens with them; the loads of all its
+// tokens (the token itself and the neighbour its channel group points at) are issued before the first value is used.
+// x is read with the default cache policy (every row is read again as somebody's neighbour), the outputs are streamed.
 template <typename IO, int VEC, int NMIX>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(QF_CX * QF_TY)
 void qshift_mix_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_, IO* __restrict__ o0, IO* __restrict__ o1,
-                       IO* __restrict__ o2, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid_tokens)
+                       IO* __restrict__ o2, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid_tokens,
+                       int tokens_per_wg)
 {
-    const int cv = blockIdx.x * blockDim.x + threadIdx.x;       // channel vector
-    const int c = cv * VEC;
-    if (c >= C) return;
-    const int t = blockIdx.y, b = blockIdx.z;
-    const size_t row = ((size_t)b * T + t) * C;
-    float xs[VEC], xx[VEC];
-    load_vec<IO, VEC>(x_ + row + c, xs);
-    // direction of this channel vector (host guarantees a vector never straddles a quarter boundary)
+    const int cx = threadIdx.x % QF_CX, ty = threadIdx.x / QF_CX;
+    const int c = (blockIdx.x * QF_CX + cx) * VEC;
+    if (c >= C) return;                                        // no barrier below
+    const int b = blockIdx.z;
+    const int t_begin = blockIdx.y * tokens_per_wg, t_end = min(T, t_begin + tokens_per_wg);
+    // direction of this channel vector (the host guarantees a vector never straddles a group boundary)
     const int cq = head_dim > 0 ? c % head_dim : c;
     const int dir = (g > 0 && cq < 4 * g) ? cq / g : 4;
-    bool have = true;
-    int ts = t;
-    if (t >= n_grid_tokens) {
-        // trailing class token (q_shift_multihead with_cls_token): passed through
-    } else if (dir < 4) {
-        const int yy = t / Wp, xc = t % Wp;
-        int sy = yy, sx = xc;
-        if (dir == 0) sx = xc - shift; else if (dir == 1) sx = xc + shift;
-        else if (dir == 2) sy = yy - shift; else sy = yy + shift;
-        have = sx >= 0 && sx < Wp && sy >= 0 && sy < Hp;
-        ts = sy * Wp + sx;
-    }
-    if (have && ts != t) load_vec<IO, VEC>(x_ + ((size_t)b * T + ts) * C + c, xx);
-    else {
+    float mu[NMIX][VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) xx[e] = have ? xs[e] : 0.f;
+    for (int m = 0; m < NMIX; ++m)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) mu[m][e] = mix_[(size_t)m * C + c + e];
+    const size_t slab = (size_t)b * T * C + c;
+    float xs[QF_TPT][VEC], xx[QF_TPT][VEC];
+    bool have[QF_TPT];
+#pragma unroll
+    for (int i = 0; i < QF_TPT; ++i) {
+        const int t = t_begin + ty + QF_TY * i;
+        have[i] = false;
+        if (t >= t_end) continue;
+        int ts = t;
+        have[i] = true;
+        if (t < n_grid_tokens && dir < 4) {                    // a trailing class token and channels >= 4g pass through
+            const int yy = t / Wp, xc = t % Wp;
+            int sy = yy, sx = xc;
+            if (dir == 0) sx = xc - shift; else if (dir == 1) sx = xc + shift;
+            else if (dir == 2) sy = yy - shift; else sy = yy + shift;
+            have[i] = sx >= 0 && sx < Wp && sy >= 0 && sy < Hp;
+            ts = have[i] ? sy * Wp + sx : t;                   // outside the grid: read the token itself, masked below
+        }
+        load_vec<IO, VEC>(x_ + slab + (size_t)t * C, xs[i]);
+        load_vec<IO, VEC>(x_ + slab + (size_t)ts * C, xx[i]);
     }
     IO* outs[3] = {o0, o1, o2};
 #pragma unroll
-    for (int m = 0; m < NMIX; ++m) {
-        float r[VEC];
+    for (int i = 0; i < QF_TPT; ++i) {
+        const int t = t_begin + ty + QF_TY * i;
+        if (t >= t_end) continue;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const float mu = mix_[(size_t)m * C + c + e];
-            r[e] = xs[e] * mu + xx[e] * (1.f - mu);
+        for (int e = 0; e < VEC; ++e) xx[i][e] = have[i] ? xx[i][e] : 0.f;      // zero fill outside the grid
+#pragma unroll
+        for (int m = 0; m < NMIX; ++m) {
+            float r[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = xs[i][e] * mu[m][e] + xx[i][e] * (1.f - mu[m][e]);
+            if constexpr (sizeof(IO) * VEC == 16) store_vec_nt<IO, VEC>(outs[m] + slab + (size_t)t * C, r);
+            else store_vec<IO, VEC>(outs[m] + slab + (size_t)t * C, r);
         }
-        store_vec<IO, VEC>(outs[m] + row + c, r);
     }
 }
 
@@ -180,7 +199,7 @@ int launch_bwd(const void* x, const float* mix, const void* const* gout, void* g
     }
     // gmix[m][c] = sum over the B * n_tchunk partial rows: the rows are (n_mix * C) wide
     const int wide = n_mix * C;
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gmix, (const float*)nullptr,
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, part, gmix, (const float*)nullptr,
                        (float*)nullptr, B * n_tchunk, wide);
     return check_launch("qshift_mix_bwd");
 }
@@ -199,16 +218,19 @@ template <typename IO, int VEC>
 int launch(const void* x, const float* mix, void* const* out, int n_mix, int B, int T, int C, int Hp, int Wp,
            int shift, int g, int head_dim, int n_grid, hipStream_t st) {
     const int ncv = C / VEC;
-    const dim3 block(ncv < 256 ? ((ncv + 63) / 64) * 64 : 256);
-    const dim3 grid((ncv + block.x - 1) / block.x, T, B);
+    // token chunks of at most QF_TY * QF_TPT tokens, evened out (196 tokens: seven chunks of 28)
+    const int n_tchunk = (T + QF_TY * QF_TPT - 1) / (QF_TY * QF_TPT);
+    const int tpw = (T + n_tchunk - 1) / n_tchunk;
+    const dim3 block(QF_CX * QF_TY);
+    const dim3 grid((ncv + QF_CX - 1) / QF_CX, n_tchunk, B);
     const IO* xx = static_cast<const IO*>(x);
     IO* o0 = static_cast<IO*>(out[0]);
     IO* o1 = n_mix > 1 ? static_cast<IO*>(out[1]) : nullptr;
     IO* o2 = n_mix > 2 ? static_cast<IO*>(out[2]) : nullptr;
     switch (n_mix) {
-        case 1: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid); break;
-        case 2: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid); break;
-        case 3: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid); break;
+        case 1: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
+        case 2: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
+        case 3: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
     }
     return check_launch("qshift_mix");
 }

@@ -27,83 +27,140 @@ namespace {
 enum { PRE_NONE = 0, PRE_RELU_SQ = 1 };
 enum { POST_NONE = 0, POST_SIGMOID_GATE = 1, POST_RESIDUAL = 2 };
 
+// Sum over the 64 lanes, the same value in every lane: four DPP steps inside each row of 16 lanes (quad swaps, half-row
+// and row mirrors), then the four row sums through scalar registers.  All lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, WAVE);
-    return x;
+    x = dpp_add<0xB1>(x);      // quad_perm [1,0,3,2]
+    x = dpp_add<0x4E>(x);      // quad_perm [2,3,0,1]
+    x = dpp_add<0x141>(x);     // row_half_mirror
+    x = dpp_add<0x140>(x);     // row_mirror
+    const int xi = __builtin_bit_cast(int, x);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0)),
+                r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16)),
+                r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32)),
+                r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
+    return (r0 + r1) + (r2 + r3);
 }
 
-template <typename IO, int VPL, int PRE, int POST, bool HAS_LN>
+// W waves share a row (1: a wave per row, short rows; 4: the workgroup's four waves, long rows), a thread keeps VPL
+// 16-byte vectors of it.  A group takes R rows whose loads are all issued before the first value is used, so a thread
+// has 2 x 16 bytes x VPL x R in flight; workgroups are short and many, the dispatcher evens out the load.
+template <int VPL> constexpr int rows_per_group_fwd() { return VPL <= 2 ? 2 : 1; }
+
+template <typename IO, int VPL, int W, int PRE, int POST, bool HAS_LN>
 __global__ __launch_bounds__(256)
 void rowfuse_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_, const IO* __restrict__ lnw_,
                     const IO* __restrict__ lnb_, const IO* __restrict__ gamma_, IO* __restrict__ out_,
                     long long rows, int N, float eps)
 {
     constexpr int V = 16 / (int)sizeof(IO);
+    constexpr int R = rows_per_group_fwd<VPL>();
+    constexpr int GROUP = WAVE * W;                            // threads per row
+    __shared__ float s_red[W > 1 ? 2 * R : 1][4];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
-    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
-    if (row >= rows) return;                                  // whole waves leave; there is no barrier below
-    const IO* a = a_ + row * N;
+    const int tid = W == 1 ? lane : (int)threadIdx.x;
     const int nvec = N / V;
-    float x[VPL][V];
-    float s = 0.f;
+    const bool has_gamma = POST == POST_RESIDUAL && gamma_ != nullptr;
+    const long long row0 = (W == 1 ? (long long)blockIdx.x * (blockDim.x >> 6) + wave : (long long)blockIdx.x) * R;
+    if (row0 >= rows) return;                                 // whole waves (W = 1) or whole workgroups (W = 4) leave
+    // the sum over a row's threads, the same value in all of them; `slot` is used once per kernel
+    auto group_sum = [&](float v, int slot) -> float {
+        v = wave_sum(v);
+        if constexpr (W > 1) {
+            if (lane == 0) s_red[slot][wave] = v;
+            __syncthreads();
+            v = (s_red[slot][0] + s_red[slot][1]) + (s_red[slot][2] + s_red[slot][3]);
+        }
+        return v;
+    };
+    // every load is issued before the first value is used: the rows and `other` are streamed (non-temporal), the
+    // per-channel vectors come from the caches; a vector waits in four registers and is widened where it is used
+    nt_u32x4 a_raw[R][VPL], o_raw[R][VPL], w_raw[VPL], b_raw[VPL], g_raw[VPL];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const bool row_ok = row0 + j < rows;                  // uniform over the group
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = tid + GROUP * i;
+            a_raw[j][i] = o_raw[j][i] = nt_u32x4{0u, 0u, 0u, 0u};
+            if (row_ok && vi < nvec) {
+                const size_t off = (size_t)(row0 + j) * N + (size_t)vi * V;
+                a_raw[j][i] = load_raw16<true>(a_ + off);
+                if (POST != POST_NONE) o_raw[j][i] = load_raw16<true>(other_ + off);
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
-        const int vi = lane + WAVE * i;
+        const int vi = tid + GROUP * i;
+        w_raw[i] = b_raw[i] = g_raw[i] = nt_u32x4{0u, 0u, 0u, 0u};
         if (vi < nvec) {
-            load_vec<IO, V>(a + (size_t)vi * V, x[i]);
+            const size_t c = (size_t)vi * V;
+            if (HAS_LN) { w_raw[i] = load_raw16<false>(lnw_ + c); b_raw[i] = load_raw16<false>(lnb_ + c); }
+            if (has_gamma) g_raw[i] = load_raw16<false>(gamma_ + c);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const long long row = row0 + j;
+        if (row >= rows) break;                               // uniform over the group
+        float x[VPL][V];
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            widen_raw16<IO, V>(a_raw[j][i], x[i]);            // threads past the row hold zeros
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 if (PRE == PRE_RELU_SQ) { const float r = fmaxf(x[i][e], 0.f); x[i][e] = r * r; }
                 s += x[i][e];
             }
-        } else {
-#pragma unroll
-            for (int e = 0; e < V; ++e) x[i][e] = 0.f;
         }
-    }
-    float mean = 0.f, rstd = 1.f;
-    if (HAS_LN) {
-        mean = wave_sum(s) / (float)N;
-        float q = 0.f;
-#pragma unroll
-        for (int i = 0; i < VPL; ++i)
-            if (lane + WAVE * i < nvec) {
-#pragma unroll
-                for (int e = 0; e < V; ++e) { const float d = x[i][e] - mean; q = fmaf(d, d, q); }
-            }
-        rstd = rsqrtf(wave_sum(q) / (float)N + eps);
-    }
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const int vi = lane + WAVE * i;
-        if (vi >= nvec) continue;
-        const size_t c = (size_t)vi * V;
-        float y[V];
+        float mean = 0.f, rstd = 1.f;
         if (HAS_LN) {
-            float w[V], b[V];
-            load_vec<IO, V>(lnw_ + c, w);
-            load_vec<IO, V>(lnb_ + c, b);
+            mean = group_sum(s, 2 * j) / (float)N;
+            float q = 0.f;
 #pragma unroll
-            for (int e = 0; e < V; ++e) y[e] = fmaf((x[i][e] - mean) * rstd, w[e], b[e]);
-        } else {
+            for (int i = 0; i < VPL; ++i)
+                if (tid + GROUP * i < nvec) {
 #pragma unroll
-            for (int e = 0; e < V; ++e) y[e] = x[i][e];
+                    for (int e = 0; e < V; ++e) { const float d = x[i][e] - mean; q = fmaf(d, d, q); }
+                }
+            rstd = rsqrtf(group_sum(q, 2 * j + 1) / (float)N + eps);
         }
-        if (POST != POST_NONE) {
-            float o[V];
-            load_vec<IO, V>(other_ + row * N + c, o);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = tid + GROUP * i;
+            if (vi >= nvec) continue;
+            const size_t c = (size_t)vi * V;
+            float y[V];
+            if (HAS_LN) {
+                float w[V], b[V];
+                widen_raw16<IO, V>(w_raw[i], w);
+                widen_raw16<IO, V>(b_raw[i], b);
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] = fmaf((x[i][e] - mean) * rstd, w[e], b[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] = x[i][e];
+            }
             if (POST == POST_SIGMOID_GATE) {
+                float o[V];
+                widen_raw16<IO, V>(o_raw[j][i], o);
 #pragma unroll
                 for (int e = 0; e < V; ++e) y[e] *= fast_rcp(1.f + fast_exp2(-o[e] * LOG2E));
-            } else {
-                float g[V];
-                if (gamma_) load_vec<IO, V>(gamma_ + c, g);
+            } else if (POST == POST_RESIDUAL) {
+                float o[V], gm[V];
+                widen_raw16<IO, V>(o_raw[j][i], o);
+                widen_raw16<IO, V>(g_raw[i], gm);
 #pragma unroll
-                for (int e = 0; e < V; ++e) y[e] = gamma_ ? fmaf(g[e], y[e], o[e]) : o[e] + y[e];
+                for (int e = 0; e < V; ++e) y[e] = has_gamma ? fmaf(gm[e], y[e], o[e]) : o[e] + y[e];
             }
+            store_vec_nt<IO, V>(out_ + row * N + c, y);
         }
-        store_vec<IO, V>(out_ + row * N + c, y);
     }
 }
 
@@ -123,16 +180,18 @@ void rowfuse_bwd_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
     const int nvec = N / V;
     constexpr int PV = SUMS ? VPL : 1, PE = SUMS ? V : 1;     // the per-channel arrays exist only with SUMS
-    float w[PV][PE], b[PV][PE], gam[PV][PE], acc_w[PV][PE], acc_b[PV][PE], acc_g[PV][PE];
+    float acc_w[PV][PE], acc_b[PV][PE], acc_g[PV][PE];
+    nt_u32x4 w_raw[PV], b_raw[PV], gam_raw[PV];              // the per-channel vectors stay packed, widened per row
 #pragma unroll
     for (int i = 0; i < PV; ++i) {
         const int vi = lane + WAVE * i;
         const bool ok = vi < nvec;
 #pragma unroll
-        for (int e = 0; e < PE; ++e) { w[i][e] = 1.f; b[i][e] = 0.f; gam[i][e] = 1.f; acc_w[i][e] = acc_b[i][e] = acc_g[i][e] = 0.f; }
+        for (int e = 0; e < PE; ++e) acc_w[i][e] = acc_b[i][e] = acc_g[i][e] = 0.f;
+        w_raw[i] = b_raw[i] = gam_raw[i] = nt_u32x4{0u, 0u, 0u, 0u};
         if constexpr (SUMS) {
-            if (ok && has_ln) { load_vec<IO, V>(lnw_ + (size_t)vi * V, w[i]); load_vec<IO, V>(lnb_ + (size_t)vi * V, b[i]); }
-            if (ok && has_gamma) load_vec<IO, V>(gamma_ + (size_t)vi * V, gam[i]);
+            if (ok && has_ln) { w_raw[i] = load_raw16<false>(lnw_ + (size_t)vi * V); b_raw[i] = load_raw16<false>(lnb_ + (size_t)vi * V); }
+            if (ok && has_gamma) gam_raw[i] = load_raw16<false>(gamma_ + (size_t)vi * V);
         }
     }
     const long long row0 = ((long long)blockIdx.x * (blockDim.x >> 6) + wave) * rows_per_wave;
@@ -168,89 +227,109 @@ void rowfuse_bwd_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_
         }
         return;
     }
-    for (int rr = 0; rr < rows_per_wave; ++rr) {
-        const long long row = row0 + rr;
-        if (row >= rows) break;                               // wave-uniform
-        float r[VPL][V], z[VPL][V], g[VPL][V], o[VPL][V];
-        float s = 0.f;
+    // The rows of a wave go in batches of RB whose loads (a, the incoming gradient, and `other` where the gate needs it)
+    // are all issued before the first value is used; a vector waits in four registers and is widened where it is used.
+    constexpr int RB = VPL == 1 ? 4 : VPL == 2 ? 2 : 1;
+    const bool need_o = post == POST_SIGMOID_GATE;            // the residual's backward does not read `other`
+    for (int rb = 0; rb < rows_per_wave; rb += RB) {
+        if (row0 + rb >= rows) break;                         // wave-uniform
+        nt_u32x4 a_raw[RB][VPL], g_raw[RB][VPL], o_raw[RB][VPL];
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) {
-            const int vi = lane + WAVE * i;
-            if (vi < nvec) {
-                const size_t off = (size_t)row * N + (size_t)vi * V;
-                load_vec<IO, V>(a_ + off, r[i]);
-                load_vec<IO, V>(g_ + off, g[i]);
-                if (post != POST_NONE) load_vec<IO, V>(other_ + off, o[i]);
+        for (int j = 0; j < RB; ++j) {
+            const bool row_ok = rb + j < rows_per_wave && row0 + rb + j < rows;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int vi = lane + WAVE * i;
+                a_raw[j][i] = g_raw[j][i] = o_raw[j][i] = nt_u32x4{0u, 0u, 0u, 0u};
+                if (row_ok && vi < nvec) {
+                    const size_t off = (size_t)(row0 + rb + j) * N + (size_t)vi * V;
+                    a_raw[j][i] = load_raw16<true>(a_ + off);
+                    g_raw[j][i] = load_raw16<true>(g_ + off);
+                    if (need_o) o_raw[j][i] = load_raw16<true>(other_ + off);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RB; ++j) {
+            const long long row = row0 + rb + j;
+            if (rb + j >= rows_per_wave || row >= rows) break;    // wave-uniform
+            float r[VPL][V], z[VPL][V], g[VPL][V];
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                widen_raw16<IO, V>(a_raw[j][i], r[i]);        // lanes past the row hold zeros
+                widen_raw16<IO, V>(g_raw[j][i], g[i]);
 #pragma unroll
                 for (int e = 0; e < V; ++e) {
                     if (pre == PRE_RELU_SQ) { r[i][e] = fmaxf(r[i][e], 0.f); z[i][e] = r[i][e] * r[i][e]; }
                     else z[i][e] = r[i][e];
                     s += z[i][e];
                 }
-            } else {
-#pragma unroll
-                for (int e = 0; e < V; ++e) { r[i][e] = z[i][e] = g[i][e] = o[i][e] = 0.f; }
             }
-        }
-        float mean = 0.f, rstd = 1.f;
-        if (has_ln) {
-            mean = wave_sum(s) / (float)N;
-            float q = 0.f;
+            float mean = 0.f, rstd = 1.f;
+            if (has_ln) {
+                mean = wave_sum(s) / (float)N;
+                float q = 0.f;
 #pragma unroll
-            for (int i = 0; i < VPL; ++i)
-                if (lane + WAVE * i < nvec) {
+                for (int i = 0; i < VPL; ++i)
+                    if (lane + WAVE * i < nvec) {
 #pragma unroll
-                    for (int e = 0; e < V; ++e) { const float d = z[i][e] - mean; q = fmaf(d, d, q); }
-                }
-            rstd = rsqrtf(wave_sum(q) / (float)N + eps);
-        }
-        // z becomes xh (normalised) under LayerNorm; g becomes gy
-        float t1 = 0.f, t2 = 0.f;
-#pragma unroll
-        for (int i = 0; i < VPL; ++i) {
-            const int vi = lane + WAVE * i;
-            if (vi >= nvec) continue;
-            float go[V];
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-                const int pi = SUMS ? i : 0, pe = SUMS ? e : 0;
-                const float xh = has_ln ? (z[i][e] - mean) * rstd : z[i][e];
-                const float y = has_ln ? fmaf(xh, w[pi][pe], b[pi][pe]) : xh;
-                float gy = g[i][e];
-                if (post == POST_SIGMOID_GATE) {
-                    const float sg = fast_rcp(1.f + fast_exp2(-o[i][e] * LOG2E));
-                    go[e] = gy * y * sg * (1.f - sg);
-                    gy *= sg;
-                } else if (post == POST_RESIDUAL) {
-                    if (has_gamma) { acc_g[pi][pe] = fmaf(gy, y, acc_g[pi][pe]); gy *= gam[pi][pe]; }
-                }
-                if (has_ln) {
-                    acc_b[pi][pe] += gy;
-                    acc_w[pi][pe] = fmaf(gy, xh, acc_w[pi][pe]);
-                    const float t = w[pi][pe] * gy;
-                    t1 += t;
-                    t2 = fmaf(t, xh, t2);
-                    g[i][e] = t;
-                } else {
-                    g[i][e] = gy;
-                }
-                z[i][e] = xh;
+                        for (int e = 0; e < V; ++e) { const float d = z[i][e] - mean; q = fmaf(d, d, q); }
+                    }
+                rstd = rsqrtf(wave_sum(q) / (float)N + eps);
             }
-            if (post == POST_SIGMOID_GATE) store_vec<IO, V>(go_ + (size_t)row * N + (size_t)vi * V, go);
-        }
-        float m1 = 0.f, m2 = 0.f;
-        if (has_ln) { m1 = wave_sum(t1) / (float)N; m2 = wave_sum(t2) / (float)N; }
+            // z becomes xh (normalised) under LayerNorm; g becomes gy
+            float t1 = 0.f, t2 = 0.f;
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) {
-            const int vi = lane + WAVE * i;
-            if (vi >= nvec) continue;
-            float ga[V];
+            for (int i = 0; i < VPL; ++i) {
+                const int vi = lane + WAVE * i;
+                if (vi >= nvec) continue;
+                float go[V], o[V], w[V], b[V], gam[V];
+                if (need_o) widen_raw16<IO, V>(o_raw[j][i], o);
+                widen_raw16<IO, V>(w_raw[SUMS ? i : 0], w);
+                widen_raw16<IO, V>(b_raw[SUMS ? i : 0], b);
+                widen_raw16<IO, V>(gam_raw[SUMS ? i : 0], gam);
 #pragma unroll
-            for (int e = 0; e < V; ++e) {
-                const float gz = has_ln ? rstd * (g[i][e] - m1 - z[i][e] * m2) : g[i][e];
-                ga[e] = pre == PRE_RELU_SQ ? gz * 2.f * r[i][e] : gz;
+                for (int e = 0; e < V; ++e) {
+                    const int pi = SUMS ? i : 0, pe = SUMS ? e : 0;
+                    const float xh = has_ln ? (z[i][e] - mean) * rstd : z[i][e];
+                    const float y = has_ln ? fmaf(xh, w[e], b[e]) : xh;
+                    float gy = g[i][e];
+                    if (post == POST_SIGMOID_GATE) {
+                        const float sg = fast_rcp(1.f + fast_exp2(-o[e] * LOG2E));
+                        go[e] = gy * y * sg * (1.f - sg);
+                        gy *= sg;
+                    } else if (post == POST_RESIDUAL) {
+                        if (has_gamma) { acc_g[pi][pe] = fmaf(gy, y, acc_g[pi][pe]); gy *= gam[e]; }
+                    }
+                    if (has_ln) {
+                        acc_b[pi][pe] += gy;
+                        acc_w[pi][pe] = fmaf(gy, xh, acc_w[pi][pe]);
+                        const float t = w[e] * gy;
+                        t1 += t;
+                        t2 = fmaf(t, xh, t2);
+                        g[i][e] = t;
+                    } else {
+                        g[i][e] = gy;
+                    }
+                    z[i][e] = xh;
+                }
+                if (post == POST_SIGMOID_GATE) store_vec_nt<IO, V>(go_ + (size_t)row * N + (size_t)vi * V, go);
             }
-            store_vec<IO, V>(ga_ + (size_t)row * N + (size_t)vi * V, ga);
+            float m1 = 0.f, m2 = 0.f;
+            if (has_ln) { m1 = wave_sum(t1) / (float)N; m2 = wave_sum(t2) / (float)N; }
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int vi = lane + WAVE * i;
+                if (vi >= nvec) continue;
+                float ga[V];
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float gz = has_ln ? rstd * (g[i][e] - m1 - z[i][e] * m2) : g[i][e];
+                    ga[e] = pre == PRE_RELU_SQ ? gz * 2.f * r[i][e] : gz;
+                }
+                store_vec_nt<IO, V>(ga_ + (size_t)row * N + (size_t)vi * V, ga);
+            }
         }
     }
     if constexpr (SUMS) {
@@ -295,7 +374,7 @@ int launch_bwd_vpl(const void* a, const void* other, const void* lnw, const void
                        static_cast<IO*>(ga), static_cast<IO*>(go), part, rows, N, eps, pre, post, rpw);
     if (SUMS) {
         const int wide = 3 * N;                               // gparam: (3, N) = g_weight, g_bias, g_gamma
-        hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + 15) / 16), dim3(256), 0, st, part, gparam,
+        hipLaunchKernelGGL(batch_sum_kernel, dim3((wide + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, part, gparam,
                            (const float*)nullptr, (float*)nullptr, (int)nblk, wide);
     }
     return check_launch("rowfuse_bwd");
@@ -322,22 +401,23 @@ int launch_bwd_io(const void* a, const void* other, const void* lnw, const void*
 #undef VRWKV_BWD
 }
 
-template <typename IO, int VPL, int PRE, int POST>
+template <typename IO, int VPL, int W, int PRE, int POST>
 int launch_ln(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
               long long rows, int N, float eps, hipStream_t st) {
-    const dim3 block(256), grid((unsigned)((rows + 3) / 4));
+    constexpr int per_wg = (W == 1 ? 4 : 1) * rows_per_group_fwd<VPL>();
+    const dim3 block(256), grid((unsigned)((rows + per_wg - 1) / per_wg));
     const IO *pa = static_cast<const IO*>(a), *po = static_cast<const IO*>(other), *pw = static_cast<const IO*>(lnw),
              *pb = static_cast<const IO*>(lnb), *pg = static_cast<const IO*>(gamma);
     IO* pout = static_cast<IO*>(out);
-    if (lnw) hipLaunchKernelGGL((rowfuse_kernel<IO, VPL, PRE, POST, true>), grid, block, 0, st, pa, po, pw, pb, pg, pout, rows, N, eps);
-    else     hipLaunchKernelGGL((rowfuse_kernel<IO, VPL, PRE, POST, false>), grid, block, 0, st, pa, po, pw, pb, pg, pout, rows, N, eps);
+    if (lnw) hipLaunchKernelGGL((rowfuse_kernel<IO, VPL, W, PRE, POST, true>), grid, block, 0, st, pa, po, pw, pb, pg, pout, rows, N, eps);
+    else     hipLaunchKernelGGL((rowfuse_kernel<IO, VPL, W, PRE, POST, false>), grid, block, 0, st, pa, po, pw, pb, pg, pout, rows, N, eps);
     return check_launch("rowfuse");
 }
 
-template <typename IO, int VPL>
+template <typename IO, int VPL, int W>
 int launch_ops(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
                long long rows, int N, int pre, int post, float eps, hipStream_t st) {
-#define VRWKV_ROW(PRE, POST) return launch_ln<IO, VPL, PRE, POST>(a, other, lnw, lnb, gamma, out, rows, N, eps, st)
+#define VRWKV_ROW(PRE, POST) return launch_ln<IO, VPL, W, PRE, POST>(a, other, lnw, lnb, gamma, out, rows, N, eps, st)
     if (pre == PRE_NONE) {
         if (post == POST_NONE) VRWKV_ROW(PRE_NONE, POST_NONE);
         if (post == POST_SIGMOID_GATE) VRWKV_ROW(PRE_NONE, POST_SIGMOID_GATE);
@@ -353,12 +433,13 @@ template <typename IO>
 int launch_io(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
               long long rows, int N, int pre, int post, float eps, hipStream_t st) {
     constexpr int V = 16 / (int)sizeof(IO);
-    const int per_lane = (N / V + WAVE - 1) / WAVE;           // 16-byte vectors a lane keeps
-    if (per_lane <= 1) return launch_ops<IO, 1>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
-    if (per_lane <= 2) return launch_ops<IO, 2>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
-    if (per_lane <= 4) return launch_ops<IO, 4>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
-    if (per_lane <= 8) return launch_ops<IO, 8>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
-    return launch_ops<IO, 16>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
+    const int nvec = N / V;
+    // rows of up to 128 vectors: a wave per row; longer ones: the four waves of a workgroup per row
+    if (nvec <= WAVE)     return launch_ops<IO, 1, 1>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
+    if (nvec <= 2 * WAVE) return launch_ops<IO, 2, 1>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
+    if (nvec <= 4 * WAVE) return launch_ops<IO, 1, 4>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
+    if (nvec <= 8 * WAVE) return launch_ops<IO, 2, 4>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
+    return launch_ops<IO, 4, 4>(a, other, lnw, lnb, gamma, out, rows, N, pre, post, eps, st);
 }
 
 }  // namespace

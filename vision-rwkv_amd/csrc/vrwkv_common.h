@@ -13,6 +13,7 @@ namespace vrwkv {
 void set_error(const char* fmt, ...);
 // Returns VRWKV_OK, or VRWKV_LAUNCH_FAILED after recording hipGetLastError()'s text.
 int check_launch(const char* what);
+int device_cus();                 // compute units of the current device (256 when the query fails)
 
 // Tuning / testing switches (0 = default behaviour).  Their initial values come from the environment variables
 // VRWKV_<NAME IN CAPITALS>, read once per process; vrwkv_set_option changes them afterwards.
@@ -68,6 +69,40 @@ __device__ __forceinline__ void store_vec(IO* __restrict__ p, const float (&in)[
     R raw;
     __builtin_memcpy(&raw, tmp, sizeof(raw));
     *reinterpret_cast<R*>(p) = raw;
+}
+// The same with the non-temporal cache policy, for tensors that are streamed through once (16-byte vectors only).
+typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+template <typename IO, int VEC>
+__device__ __forceinline__ void load_vec_nt(const IO* __restrict__ p, float (&out)[VEC]) {
+    static_assert(sizeof(IO) * VEC == 16, "16-byte vectors");
+    const nt_u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p));
+    IO tmp[VEC];
+    __builtin_memcpy(tmp, &raw, sizeof(raw));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) out[e] = to_f32(tmp[e]);
+}
+// A 16-byte vector fetched now and widened where it is used (keeps four registers, not VEC, while it waits).
+template <bool NT>
+__device__ __forceinline__ nt_u32x4 load_raw16(const void* p) {
+    return NT ? __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p)) : *reinterpret_cast<const nt_u32x4*>(p);
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void widen_raw16(nt_u32x4 raw, float (&out)[VEC]) {
+    static_assert(sizeof(IO) * VEC == 16, "16-byte vectors");
+    IO tmp[VEC];
+    __builtin_memcpy(tmp, &raw, sizeof(raw));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) out[e] = to_f32(tmp[e]);
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void store_vec_nt(IO* __restrict__ p, const float (&in)[VEC]) {
+    static_assert(sizeof(IO) * VEC == 16, "16-byte vectors");
+    IO tmp[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) tmp[e] = from_f32<IO>(in[e]);
+    nt_u32x4 raw;
+    __builtin_memcpy(&raw, tmp, sizeof(raw));
+    __builtin_nontemporal_store(raw, reinterpret_cast<nt_u32x4*>(p));
 }
 // Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait
 // for outstanding global loads/stores (vmcnt), so prefetches stay in flight across it.
@@ -133,20 +168,34 @@ __device__ __forceinline__ void stamp(int wave, int slot, int point) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// out[c] = sum_b part[b*C + c] for up to two (part, out) pairs (the second may be null).  256 threads =
-// 16 channels x 16 slices of the batch, so the B loads of a channel are issued 16 at a time instead of
-// one after the other; fixed summation order (deterministic).  Grid: ceil(C / 16).
-__global__ inline void batch_sum_kernel(const float* __restrict__ part0, float* __restrict__ out0,
-                                        const float* __restrict__ part1, float* __restrict__ out1, int B, int C) {
-    __shared__ float red[2][16][17];
-    const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
-    const int c = blockIdx.x * 16 + cl;
+// out[c] = sum_b part[b*C + c] for up to two (part, out) pairs (the second may be null).  1024 threads = 64 columns
+// (one 256-byte piece of a row per wave load) x 16 slices of the batch, eight loads of a slice in flight at a time;
+// the slices are added in a fixed order (deterministic).  Grid: ceil(C / 64), block: BATCH_SUM_THREADS.
+constexpr int BATCH_SUM_THREADS = 1024, BATCH_SUM_COLS = 64;
+__global__ __launch_bounds__(1024) inline void batch_sum_kernel(const float* __restrict__ part0, float* __restrict__ out0,
+                                                                const float* __restrict__ part1, float* __restrict__ out1,
+                                                                int B, int C) {
+    __shared__ float red[2][16][BATCH_SUM_COLS];
+    const int cl = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int c = blockIdx.x * BATCH_SUM_COLS + cl;
     float s0 = 0.f, s1 = 0.f;
-    if (c < C)
-        for (int b = slice; b < B; b += 16) {
+    if (c < C) {
+        int b = slice;
+        for (; b + 16 * 7 < B; b += 16 * 8) {
+            float t0[8], t1[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                t0[i] = part0[(size_t)(b + 16 * i) * C + c];
+                t1[i] = part1 ? part1[(size_t)(b + 16 * i) * C + c] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { s0 += t0[i]; s1 += t1[i]; }
+        }
+        for (; b < B; b += 16) {
             s0 += part0[(size_t)b * C + c];
             if (part1) s1 += part1[(size_t)b * C + c];
         }
+    }
     red[0][slice][cl] = s0;
     red[1][slice][cl] = s1;
     __syncthreads();

@@ -265,7 +265,7 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
 #undef VRWKV_SCAN
             hipLaunchKernelGGL((wkv6_bwd_fallback<IO, WT, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, gr, gk, gv, gw,
                                a, gu_part, todo, T, C, H);
-            hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gu_part, gu, (const float*)nullptr,
+            hipLaunchKernelGGL(batch_sum_kernel, dim3((C + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, gu_part, gu, (const float*)nullptr,
                                (float*)nullptr, B, C);
             return check_launch("wkv6_bwd (chunked)");
         }
@@ -277,7 +277,7 @@ int launch_all(const void* r, const void* k, const void* v, const void* w, const
     hipLaunchKernelGGL((wkv6_bwd_sweep_s<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, gr, a, gu_part, T, C, H);
     hipLaunchKernelGGL((wkv6_bwd_sweep_g<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, vv, ww, u, gy, a, gk, gw, T, C, H);
     hipLaunchKernelGGL((wkv6_bwd_sweep_v<IO, WT, 0, EW>), grid, block, 0, st, rr, kk, ww, u, gy, gv, T, C, H);
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + 15) / 16), dim3(256), 0, st, gu_part, gu, (const float*)nullptr, (float*)nullptr, B, C);   // torch.sum(gu, 0), vrwkv6.py:69
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((C + BATCH_SUM_COLS - 1) / BATCH_SUM_COLS), dim3(BATCH_SUM_THREADS), 0, st, gu_part, gu, (const float*)nullptr, (float*)nullptr, B, C);   // torch.sum(gu, 0), vrwkv6.py:69
     return check_launch("wkv6_bwd");
 }
 
