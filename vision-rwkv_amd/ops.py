@@ -109,10 +109,11 @@ class WKV(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, w, u, k, v):
-        ctx.save_for_backward(w, u, k, v)
         out_dtype = w.dtype if w.dtype in (torch.half, torch.bfloat16) else torch.float32
         wf = w.float().contiguous()
         uf = u.float().contiguous()
+        ctx.save_for_backward(wf, uf, k, v)                # the fp32 copies serve the backward too
+        ctx.out_dtype = out_dtype
         if k.dtype == out_dtype and v.dtype == out_dtype:
             return bi_wkv_forward(wf, uf, k.contiguous(), v.contiguous())
         y = bi_wkv_forward(wf, uf, k.float().contiguous(), v.float().contiguous())
@@ -121,10 +122,8 @@ class WKV(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gy):
         # vrwkv.py:47-61: gradients in fp32, returned in w's dtype when that is half / bfloat16
-        w, u, k, v = ctx.saved_tensors
-        out_dtype = w.dtype if w.dtype in (torch.half, torch.bfloat16) else torch.float32
-        wf = w.float().contiguous()
-        uf = u.float().contiguous()
+        wf, uf, k, v = ctx.saved_tensors
+        out_dtype = ctx.out_dtype
         if k.dtype == out_dtype and v.dtype == out_dtype and out_dtype != torch.float32:
             gw, gu, gk, gv = bi_wkv_backward(wf, uf, k.contiguous(), v.contiguous(), gy.to(out_dtype).contiguous())
         else:
@@ -132,7 +131,8 @@ class WKV(torch.autograd.Function):
                                              gy.float().contiguous())
         if out_dtype == torch.float32:
             return (gw, gu, gk, gv)
-        return (gw.to(out_dtype), gu.to(out_dtype), gk.to(out_dtype), gv.to(out_dtype))
+        gwu = torch.stack((gw, gu)).to(out_dtype)           # one cast for both parameter gradients
+        return (gwu[0], gwu[1], gk.to(out_dtype), gv.to(out_dtype))
 
 
 class _WKVLegacy(torch.autograd.Function):
@@ -383,9 +383,10 @@ class _RowFuse(torch.autograd.Function):
                                            gout.data_ptr(), ga.data_ptr(), ptr(go), ptr(gparam), rows, N, pre, post,
                                            float(eps), _DT[a.dtype], ptr(ws), ws_bytes, _stream_ptr(a.device)))
         g_other = go if post == POST_SIGMOID_GATE else (gout if post == POST_RESIDUAL else None)
-        g_w = gparam[0].to(ln_weight.dtype) if ln_weight is not None else None
-        g_b = gparam[1].to(ln_bias.dtype) if ln_bias is not None else None
-        g_g = gparam[2].to(gamma.dtype) if (gamma is not None and post == POST_RESIDUAL) else None
+        gp = gparam.to(a.dtype) if sums else None            # one cast for the three parameter gradients
+        g_w = gp[0] if ln_weight is not None else None
+        g_b = gp[1] if ln_bias is not None else None
+        g_g = gp[2] if (gamma is not None and post == POST_RESIDUAL) else None
         return ga, g_other, g_w, g_b, g_g, None, None, None
 
 
@@ -614,7 +615,7 @@ def q_shift_mix_autograd(x, mixes, shift_pixel=1, gamma=1 / 4, patch_resolution=
     _check_input(x, "x")
     if x.dim() != 3 or x.dtype not in _DT:
         raise RuntimeError("x must be (B,T,C) float32 / bfloat16 / float16")
-    table = torch.stack([m.reshape(-1).float() for m in mixes])
+    table = torch.stack([m.reshape(-1) for m in mixes]).float()       # one cast, differentiated as one
     Hp, Wp = patch_resolution
     if not _equal_quarters(x.shape[-1], gamma, head_dim):
         xx = q_shift(x, shift_pixel, gamma, patch_resolution)
