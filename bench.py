@@ -218,6 +218,137 @@ def sweep_section(torch, ops, steps, warmup):
     return rows
 
 
+def elementwise_section(torch, ops):
+    """The element-wise kernels of a block (q_shift + mixes, the row-wise epilogues, the VRWKV6 mix steps) at the
+    VRWKV-B layer shape (64, 196, 768) and the VRWKV-L one (32, 576, 1024), bf16: each timed as calls on rotating
+    buffer sets back to back (six sets, more than the last-level cache holds), in us and GB/s of the algorithmic
+    bytes against the 8 TB/s HBM figure.  Everything is called through the C ABI (at 15-30 us per kernel the host work
+    of the Python wrappers would dominate a per-call figure)."""
+    import ctypes
+    from vision_rwkv_amd import _lib
+    from vision_rwkv_amd import ops as O
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    NB = 6
+    dt = torch.bfloat16
+    es = 2
+
+    def timed(fns, reps=4):
+        for f in fns:
+            f()
+        torch.cuda.synchronize()
+        r = []
+        for _ in range(REPEATS):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                for f in fns:
+                    f()
+            e1.record()
+            torch.cuda.synchronize()
+            r.append(e0.elapsed_time(e1) / (reps * len(fns)) * 1e3)
+        return sorted(r)[len(r) // 2]
+
+    out = []
+    for (Bn, Hp, Wp, Cn) in ((64, 14, 14, 768), (32, 24, 24, 1024)):
+        Tn = Hp * Wp
+        n = Bn * Tn * Cn
+        g = torch.Generator(device="cpu").manual_seed(Cn)
+        xs = [torch.randn(Bn, Tn, Cn, generator=g).to(dev).to(dt) for _ in range(NB)]
+        os_ = [torch.randn(Bn, Tn, Cn, generator=g).to(dev).to(dt) for _ in range(NB)]
+        gs = [torch.randn(Bn, Tn, Cn, generator=g).to(dev).to(dt) for _ in range(3)]
+        mixes = [torch.rand(Cn, generator=g).to(dev) for _ in range(3)]
+        tab3 = O.stack_mixes(mixes, dev)
+        tab2 = tab3[:2].contiguous()
+        lw, lb, gm = (torch.randn(Cn, generator=g).to(dev).to(dt) for _ in range(3))
+        rows = []
+
+        def add(name, us, nbytes):
+            rows.append({"kernel": name, "us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+                         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+
+        def each(f):
+            return [(lambda i=i: f(i)) for i in range(NB)]
+
+        st = torch.cuda.current_stream().cuda_stream
+        rws = Bn * Tn
+        fptr = lambda t: ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_float))
+        outs3 = [torch.empty_like(xs[0]) for _ in range(5)]
+        optr = {k: (ctypes.c_void_p * k)(*[t.data_ptr() for t in outs3[:k]]) for k in (2, 3, 5)}
+
+        def qs_fwd(i, tab, k):
+            _lib.check(L.vrwkv_qshift_mix(xs[i].data_ptr(), fptr(tab), optr[k], k, Bn, Tn, Cn, Hp, Wp, 1, Cn // 4, 0,
+                                          _lib.VRWKV_BF16, st))
+
+        def row_fwd(a, o, w_, b_, g_, N, pre, post, out):
+            p = lambda t: t.data_ptr() if t is not None else None
+            _lib.check(L.vrwkv_rowfuse(a.data_ptr(), p(o), p(w_), p(b_), p(g_), out.data_ptr(), a.numel() // N, N, pre, post,
+                                       1e-5, _lib.VRWKV_BF16, st))
+
+        add("q_shift + 3 mixes (1 read, 3 writes)", timed(each(lambda i: qs_fwd(i, tab3, 3))), 4 * n * es)
+        add("q_shift + 2 mixes (1 read, 2 writes)", timed(each(lambda i: qs_fwd(i, tab2, 2))), 3 * n * es)
+        o1 = outs3[0]
+        add("LayerNorm + sigmoid gate (2 reads, 1 write)",
+            timed(each(lambda i: row_fwd(xs[i], os_[i], lw, lb, None, Cn, O.PRE_NONE, O.POST_SIGMOID_GATE, o1))), 3 * n * es)
+        add("sigmoid gate (2 reads, 1 write)",
+            timed(each(lambda i: row_fwd(xs[i], os_[i], None, None, None, Cn, O.PRE_NONE, O.POST_SIGMOID_GATE, o1))), 3 * n * es)
+        add("LayerNorm + layer-scaled residual (2 reads, 1 write)",
+            timed(each(lambda i: row_fwd(xs[i], os_[i], lw, lb, gm, Cn, O.PRE_NONE, O.POST_RESIDUAL, o1))), 3 * n * es)
+        x4 = [torch.randn(Bn, Tn, 4 * Cn, generator=g).to(dev).to(dt) for _ in range(3)]
+        o4 = torch.empty_like(x4[0])
+        lw4, lb4 = (torch.randn(4 * Cn, generator=g).to(dev).to(dt) for _ in range(2))
+        add("relu^2 + LayerNorm on 4C channels (1 read, 1 write)",
+            timed([(lambda i=i: row_fwd(x4[i], None, lw4, lb4, None, 4 * Cn, O.PRE_RELU_SQ, O.POST_NONE, o4)) for i in range(3)]),
+            2 * 4 * n * es)
+        del x4, o4
+        m5 = [torch.randn(5, Bn, Tn, Cn, generator=g).to(dev).to(dt) for _ in range(3)]
+        mt = O.stack_mixes([torch.rand(Cn, generator=g).to(dev) for _ in range(5)], dev)
+        add("VRWKV6 five token mixes (7 reads, 5 writes)",
+            timed([(lambda i=i: _lib.check(L.vrwkv_maa_mix(xs[i].data_ptr(), os_[i].data_ptr(), m5[i].data_ptr(), fptr(mt),
+                                                           optr[5], rws, Cn, _lib.VRWKV_BF16, st))) for i in range(3)]),
+            12 * n * es)
+        del m5
+        y32 = [torch.randn(Bn, Tn, Cn, generator=g).to(dev) for _ in range(NB)]
+        add("VRWKV6 GroupNorm x SiLU gate (fp32 y and gate read, 1 write)",
+            timed(each(lambda i: _lib.check(L.vrwkv_groupnorm_gate(y32[i].data_ptr(), os_[i].data_ptr(), lw.data_ptr(),
+                                                                   lb.data_ptr(), o1.data_ptr(), rws, Cn, 64, 1e-5,
+                                                                   _lib.VRWKV_F32, _lib.VRWKV_BF16, st)))), n * (4 + 2 * es))
+        del y32
+        ga = torch.empty_like(xs[0])
+        go = torch.empty_like(xs[0])
+        gparam = torch.empty(3, Cn, dtype=torch.float32, device=dev)
+        wsb = L.vrwkv_rowfuse_bwd_workspace_bytes(rws, Cn)
+        ws = torch.empty(max(wsb, 1), dtype=torch.uint8, device=dev)
+
+        def row_bwd(i, post, with_ln):
+            _lib.check(L.vrwkv_rowfuse_bwd(xs[i].data_ptr(), os_[i].data_ptr(), lw.data_ptr() if with_ln else None,
+                                           lb.data_ptr() if with_ln else None,
+                                           gm.data_ptr() if post == O.POST_RESIDUAL else None, gs[i % 3].data_ptr(),
+                                           ga.data_ptr(), go.data_ptr() if post == O.POST_SIGMOID_GATE else None,
+                                           ctypes.cast(gparam.data_ptr(), ctypes.POINTER(ctypes.c_float)), rws, Cn,
+                                           O.PRE_NONE, post, 1e-5, _lib.VRWKV_BF16, ws.data_ptr(), wsb, st))
+
+        add("backward of LayerNorm + layer-scaled residual (2 reads, 1 write; + reduction launch)",
+            timed(each(lambda i: row_bwd(i, O.POST_RESIDUAL, True))), 3 * n * es)
+        add("backward of sigmoid gate (3 reads, 2 writes)",
+            timed(each(lambda i: row_bwd(i, O.POST_SIGMOID_GATE, False))), 5 * n * es)
+        gx = torch.empty_like(xs[0])
+        gmix = torch.empty(3, Cn, dtype=torch.float32, device=dev)
+        qwb = L.vrwkv_qshift_mix_bwd_workspace_bytes(3, Bn, Tn, Cn)
+        qws = torch.empty(qwb, dtype=torch.uint8, device=dev)
+        gptr = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in gs])
+
+        def qs_bwd(i):
+            _lib.check(L.vrwkv_qshift_mix_bwd(xs[i].data_ptr(), ctypes.cast(tab3.data_ptr(), ctypes.POINTER(ctypes.c_float)),
+                                              gptr, 3, gx.data_ptr(), ctypes.cast(gmix.data_ptr(), ctypes.POINTER(ctypes.c_float)),
+                                              Bn, Tn, Cn, Hp, Wp, 1, Cn // 4, 0, _lib.VRWKV_BF16, qws.data_ptr(), qwb, st))
+
+        add("backward of q_shift + 3 mixes (4 reads, 1 write; + reduction launch)", timed(each(qs_bwd)), 5 * n * es)
+        out.append({"shape": [Bn, Tn, Cn], "dtype": "bf16", "kernels": rows})
+        del xs, os_, gs
+    return out
+
+
 def backbone_section(torch, ops, steps, warmup):
     """VRWKV-L forward (24 blocks, C=1024, 384x384 input -> T=576) at batch 32 in bf16, random weights:
     ms per forward, and the share of it spent in the 24 Bi-WKV calls (timed alone at the same shape)."""
@@ -313,6 +444,7 @@ def main():
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-kernel measurements")
     ap.add_argument("--no-sweep", action="store_true", help="skip the dense-prediction shape sweep (B=2, long T)")
     ap.add_argument("--no-config2", action="store_true", help="skip the B=2, T=4150, C=768 bf16 measurement")
+    ap.add_argument("--no-elementwise", action="store_true", help="skip the element-wise block kernels (q_shift + mix, row epilogues)")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -445,6 +577,8 @@ def main():
         out["config2"] = config2_section(torch, ops, 20, 10)
     if not args.no_sweep:
         out["sweep"] = sweep_section(torch, ops, 10, 3)
+    if not args.no_elementwise:
+        out["elementwise"] = elementwise_section(torch, ops)
     if not args.no_backbone:
         out["backbone"] = backbone_section(torch, ops, 5, 3)
     print(json.dumps(out))
