@@ -41,6 +41,12 @@ def _shift_and_mix(module, x, mixes, shift_pixel, patch_resolution, with_cls_tok
     return [x * m + sx * (1 - m) for m in mixes()]
 
 
+def _layer_norm(ln, x):
+    """nn.LayerNorm over the channels through the fused row kernel (forward and backward); tensor ops where it does
+    not apply."""
+    return row_fuse(x, None, ln.weight, ln.bias, None, PRE_NONE, POST_NONE, ln.eps)
+
+
 class VRWKV_SpatialMix_V6(nn.Module):
     def __init__(self, n_embd, n_head, n_layer, layer_id, shift_pixel=1, key_norm=False, with_cls_token=False,
                  fused_shift=True):
@@ -144,15 +150,15 @@ class Block6(nn.Module):
 
     def forward(self, x, patch_resolution):
         if self.layer_id == 0:
-            x = self.ln0(x)
+            x = _layer_norm(self.ln0, x)
         g1 = self.gamma1 if self.layer_scale else None
         g2 = self.gamma2 if self.layer_scale else None
         if self.post_norm:                                   # scale, add and post-norm in one pass
             x = row_fuse(self.att(x, patch_resolution), x, self.ln1.weight, self.ln1.bias, g1, PRE_NONE, POST_RESIDUAL, self.ln1.eps)
             x = row_fuse(self.ffn(x, patch_resolution), x, self.ln2.weight, self.ln2.bias, g2, PRE_NONE, POST_RESIDUAL, self.ln2.eps)
         else:
-            x = row_fuse(self.att(self.ln1(x), patch_resolution), x, None, None, g1, PRE_NONE, POST_RESIDUAL)
-            x = row_fuse(self.ffn(self.ln2(x), patch_resolution), x, None, None, g2, PRE_NONE, POST_RESIDUAL)
+            x = row_fuse(self.att(_layer_norm(self.ln1, x), patch_resolution), x, None, None, g1, PRE_NONE, POST_RESIDUAL)
+            x = row_fuse(self.ffn(_layer_norm(self.ln2, x), patch_resolution), x, None, None, g2, PRE_NONE, POST_RESIDUAL)
         return x
 
 
@@ -182,7 +188,7 @@ class VRWKV6(VRWKV):
         for layer in self.layers:
             x = layer(x, res)
         if self.final_norm:
-            x = self.ln1(x)
+            x = _layer_norm(self.ln1, x)
         C = x.shape[-1]
         patches = x[:, :-1] if self.with_cls_token else x
         fmap = patches.reshape(B, res[0], res[1], C).permute(0, 3, 1, 2)

@@ -20,6 +20,17 @@
 namespace vrwkv {
 namespace {
 
+// Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own.  A token's neighbour rows belong to the
+// next token chunk of the same image, so the launch is one-dimensional and XCD x takes a contiguous eighth of the
+// (channel block, token chunk, image) grid: an image's chunks then share an L2 and the neighbour reads hit in it.
+struct Block3 { int x, y, z; };
+__device__ __forceinline__ Block3 xcd_block(int gx, int gy, int gz) {
+    const int total = gx * gy * gz, id = blockIdx.x;
+    const int per = total / 8;
+    const int v = (total % 8 == 0) ? (id % 8) * per + id / 8 : id;
+    return Block3{v % gx, (v / gx) % gy, v / (gx * gy)};
+}
+
 constexpr int QF_CX = 32, QF_TY = 8;   // forward workgroup: 32 channel vectors x 8 token lanes
 constexpr int QF_TPT = 4;              // tokens per thread: a workgroup covers up to 32 tokens of 32 channel vectors
 
@@ -30,13 +41,14 @@ template <typename IO, int VEC, int NMIX>
 __global__ __launch_bounds__(QF_CX * QF_TY)
 void qshift_mix_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_, IO* __restrict__ o0, IO* __restrict__ o1,
                        IO* __restrict__ o2, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid_tokens,
-                       int tokens_per_wg)
+                       int tokens_per_wg, int gx, int gy, int gz)
 {
+    const Block3 blk = xcd_block(gx, gy, gz);
     const int cx = threadIdx.x % QF_CX, ty = threadIdx.x / QF_CX;
-    const int c = (blockIdx.x * QF_CX + cx) * VEC;
+    const int c = (blk.x * QF_CX + cx) * VEC;
     if (c >= C) return;                                        // no barrier below
-    const int b = blockIdx.z;
-    const int t_begin = blockIdx.y * tokens_per_wg, t_end = min(T, t_begin + tokens_per_wg);
+    const int b = blk.z;
+    const int t_begin = blk.y * tokens_per_wg, t_end = min(T, t_begin + tokens_per_wg);
     // direction of this channel vector (the host guarantees a vector never straddles a group boundary)
     const int cq = head_dim > 0 ? c % head_dim : c;
     const int dir = (g > 0 && cq < 4 * g) ? cq / g : 4;
@@ -116,14 +128,15 @@ __global__ __launch_bounds__(QS_CX * QS_TY)
 void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_, const IO* __restrict__ g0,
                            const IO* __restrict__ g1, const IO* __restrict__ g2, IO* __restrict__ gx_,
                            float* __restrict__ gmix_part, int T, int C, int Hp, int Wp, int shift, int g, int head_dim,
-                           int n_grid_tokens, int n_tchunk)
+                           int n_grid_tokens, int n_tchunk, int gx, int gz)
 {
     __shared__ float s_acc[QS_TY][NMIX][QS_CX * VEC];
+    const Block3 blk = xcd_block(gx, n_tchunk, gz);
     const int cx = threadIdx.x % QS_CX, ty = threadIdx.x / QS_CX;
-    const int cv = blockIdx.x * QS_CX + cx;
+    const int cv = blk.x * QS_CX + cx;
     const int c = cv * VEC;
     const bool cok = c < C;
-    const int tc = blockIdx.y, b = blockIdx.z;
+    const int tc = blk.y, b = blk.z;
     const int dir = qs_dir(cok ? c : 0, g, head_dim);
     const IO* gs[3] = {g0, g1, g2};
     float mu[NMIX][VEC], acc[NMIX][VEC];
@@ -132,34 +145,57 @@ void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) { mu[m][e] = cok ? mix_[(size_t)m * C + c + e] : 0.f; acc[m][e] = 0.f; }
     const size_t slab = (size_t)b * T * C + c;
+    // the chunk's tokens, evened out over the chunks (196 tokens: seven chunks of 28); a thread takes every eighth,
+    // two at a time: the sixteen loads of a pair are issued before the first value is used and wait packed
+    const int tch = (T + n_tchunk - 1) / n_tchunk;
+    const int t_begin = tc * tch, t_end = min(T, t_begin + tch);
+    using Packed = typename RawVec<sizeof(IO) * VEC>::type;
     if (cok) {
 #pragma unroll
-        for (int i = 0; i < QS_TCH / QS_TY; ++i) {
-            const int t = tc * QS_TCH + ty + QS_TY * i;
-            if (t >= T) continue;
-            const int ts = qs_src(t, dir, Hp, Wp, shift, n_grid_tokens);
-            const int td = qs_dst(t, dir, Hp, Wp, shift, n_grid_tokens);
-            // neighbours outside the grid are read from the token itself and masked: no divergent branches, so all
-            // loads of a token are in flight together
-            float xs[VEC], xx[VEC], gx[VEC], gt[NMIX][VEC], gd[NMIX][VEC];
-            load_vec<IO, VEC>(x_ + slab + (size_t)t * C, xs);
-            load_vec<IO, VEC>(x_ + slab + (size_t)(ts >= 0 ? ts : t) * C, xx);
+        for (int i0 = 0; i0 < QS_TCH / QS_TY; i0 += 2) {
+            Packed pxs[2], pxx[2], pgt[2][NMIX], pgd[2][NMIX];
+            float keep_s[2], keep_d[2];
+            int tt[2];
 #pragma unroll
-            for (int m = 0; m < NMIX; ++m) {
-                load_vec<IO, VEC>(gs[m] + slab + (size_t)t * C, gt[m]);
-                load_vec<IO, VEC>(gs[m] + slab + (size_t)(td >= 0 ? td : t) * C, gd[m]);
-            }
-            const float keep_s = ts >= 0 ? 1.f : 0.f, keep_d = td >= 0 ? 1.f : 0.f;
+            for (int j = 0; j < 2; ++j) {
+                const int t = t_begin + ty + QS_TY * (i0 + j);
+                tt[j] = t < t_end ? t : -1;
+                const int tl = t < t_end ? t : t_begin;          // a token past the chunk: load a valid one, use nothing
+                const int ts = qs_src(tl, dir, Hp, Wp, shift, n_grid_tokens);
+                const int td = qs_dst(tl, dir, Hp, Wp, shift, n_grid_tokens);
+                // neighbours outside the grid are read from the token itself and masked: no divergent branches
+                keep_s[j] = ts >= 0 ? 1.f : 0.f;
+                keep_d[j] = td >= 0 ? 1.f : 0.f;
+                pxs[j] = load_packed<IO, VEC>(x_ + slab + (size_t)tl * C);
+                pxx[j] = load_packed<IO, VEC>(x_ + slab + (size_t)(ts >= 0 ? ts : tl) * C);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
-#pragma unroll
-            for (int m = 0; m < NMIX; ++m)
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    gx[e] = fmaf(gt[m][e], mu[m][e], fmaf(keep_d * gd[m][e], 1.f - mu[m][e], gx[e]));
-                    acc[m][e] = fmaf(gt[m][e], xs[e] - keep_s * xx[e], acc[m][e]);
+                for (int m = 0; m < NMIX; ++m) {
+                    pgt[j][m] = load_packed<IO, VEC>(gs[m] + slab + (size_t)tl * C);
+                    pgd[j][m] = load_packed<IO, VEC>(gs[m] + slab + (size_t)(td >= 0 ? td : tl) * C);
                 }
-            store_vec<IO, VEC>(gx_ + slab + (size_t)t * C, gx);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (tt[j] < 0) continue;
+                float xs[VEC], xx[VEC], gx[VEC];
+                widen_packed<IO, VEC>(pxs[j], xs);
+                widen_packed<IO, VEC>(pxx[j], xx);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
+#pragma unroll
+                for (int m = 0; m < NMIX; ++m) {
+                    float gt[VEC], gd[VEC];
+                    widen_packed<IO, VEC>(pgt[j][m], gt);
+                    widen_packed<IO, VEC>(pgd[j][m], gd);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        gx[e] = fmaf(gt[e], mu[m][e], fmaf(keep_d[j] * gd[e], 1.f - mu[m][e], gx[e]));
+                        acc[m][e] = fmaf(gt[e], xs[e] - keep_s[j] * xx[e], acc[m][e]);
+                    }
+                }
+                if constexpr (sizeof(IO) * VEC == 16) store_vec_nt<IO, VEC>(gx_ + slab + (size_t)tt[j] * C, gx);
+                else store_vec<IO, VEC>(gx_ + slab + (size_t)tt[j] * C, gx);
+            }
         }
     }
     // the eight token lanes' sums of a column are added in a fixed order and written as one partial row
@@ -171,7 +207,7 @@ void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ 
     float* part = gmix_part + ((size_t)b * n_tchunk + tc) * NMIX * C;
     for (int o = threadIdx.x; o < NMIX * QS_CX * VEC; o += QS_CX * QS_TY) {
         const int m = o / (QS_CX * VEC), col = o % (QS_CX * VEC);
-        const int cg = blockIdx.x * QS_CX * VEC + col;
+        const int cg = blk.x * QS_CX * VEC + col;
         if (cg >= C) continue;
         float sum = 0.f;
 #pragma unroll
@@ -186,16 +222,21 @@ int launch_bwd(const void* x, const float* mix, const void* const* gout, void* g
     const int ncv = C / VEC;
     const int n_tchunk = (T + QS_TCH - 1) / QS_TCH;
     const dim3 block(QS_CX * QS_TY);
-    const dim3 grid((ncv + QS_CX - 1) / QS_CX, n_tchunk, B);
+    const int gbx = (ncv + QS_CX - 1) / QS_CX;
+    if ((long long)gbx * n_tchunk * B > 0x7fffffffLL) {
+        set_error("qshift_mix_bwd: too many workgroups (%d x %d x %d)", gbx, n_tchunk, B);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    const dim3 grid((unsigned)gbx * n_tchunk * B);
     const IO* xx = static_cast<const IO*>(x);
     const IO* g0 = static_cast<const IO*>(gout[0]);
     const IO* g1 = n_mix > 1 ? static_cast<const IO*>(gout[1]) : nullptr;
     const IO* g2 = n_mix > 2 ? static_cast<const IO*>(gout[2]) : nullptr;
     IO* pgx = static_cast<IO*>(gx);
     switch (n_mix) {
-        case 1: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
-        case 2: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
-        case 3: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk); break;
+        case 1: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk, gbx, B); break;
+        case 2: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk, gbx, B); break;
+        case 3: hipLaunchKernelGGL((qshift_mix_bwd_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, g0, g1, g2, pgx, part, T, C, Hp, Wp, shift, g, head_dim, n_grid, n_tchunk, gbx, B); break;
     }
     // gmix[m][c] = sum over the B * n_tchunk partial rows: the rows are (n_mix * C) wide
     const int wide = n_mix * C;
@@ -222,15 +263,20 @@ int launch(const void* x, const float* mix, void* const* out, int n_mix, int B, 
     const int n_tchunk = (T + QF_TY * QF_TPT - 1) / (QF_TY * QF_TPT);
     const int tpw = (T + n_tchunk - 1) / n_tchunk;
     const dim3 block(QF_CX * QF_TY);
-    const dim3 grid((ncv + QF_CX - 1) / QF_CX, n_tchunk, B);
+    const int gx = (ncv + QF_CX - 1) / QF_CX;
+    if ((long long)gx * n_tchunk * B > 0x7fffffffLL) {
+        set_error("qshift_mix: too many workgroups (%d x %d x %d)", gx, n_tchunk, B);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
+    const dim3 grid((unsigned)gx * n_tchunk * B);
     const IO* xx = static_cast<const IO*>(x);
     IO* o0 = static_cast<IO*>(out[0]);
     IO* o1 = n_mix > 1 ? static_cast<IO*>(out[1]) : nullptr;
     IO* o2 = n_mix > 2 ? static_cast<IO*>(out[2]) : nullptr;
     switch (n_mix) {
-        case 1: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
-        case 2: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
-        case 3: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw); break;
+        case 1: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 1>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw, gx, n_tchunk, B); break;
+        case 2: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 2>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw, gx, n_tchunk, B); break;
+        case 3: hipLaunchKernelGGL((qshift_mix_kernel<IO, VEC, 3>), grid, block, 0, st, xx, mix, o0, o1, o2, T, C, Hp, Wp, shift, g, head_dim, n_grid, tpw, gx, n_tchunk, B); break;
     }
     return check_launch("qshift_mix");
 }

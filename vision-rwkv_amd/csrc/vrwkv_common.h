@@ -70,6 +70,18 @@ __device__ __forceinline__ void store_vec(IO* __restrict__ p, const float (&in)[
     __builtin_memcpy(&raw, tmp, sizeof(raw));
     *reinterpret_cast<R*>(p) = raw;
 }
+// A vector of VEC elements fetched now and widened where it is used (it waits in its packed form).
+template <typename IO, int VEC>
+__device__ __forceinline__ typename RawVec<sizeof(IO) * VEC>::type load_packed(const IO* __restrict__ p) {
+    return *reinterpret_cast<const typename RawVec<sizeof(IO) * VEC>::type*>(p);
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void widen_packed(typename RawVec<sizeof(IO) * VEC>::type raw, float (&out)[VEC]) {
+    IO tmp[VEC];
+    __builtin_memcpy(tmp, &raw, sizeof(raw));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) out[e] = to_f32(tmp[e]);
+}
 // The same with the non-temporal cache policy, for tensors that are streamed through once (16-byte vectors only).
 typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
 template <typename IO, int VEC>
