@@ -211,7 +211,8 @@ def test_pos_embed_resize_restates_the_interpolation():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("N,dtype", [(1024, torch.bfloat16), (4096, torch.bfloat16), (768, torch.float32),
-                                     (3072, torch.float32), (64, torch.float16), (8192, torch.bfloat16)])
+                                     (3072, torch.float32), (64, torch.float16), (8192, torch.bfloat16),
+                                     (768, torch.bfloat16), (2048, torch.bfloat16), (1032, torch.bfloat16)])
 def test_row_fuse_against_oracle(N, dtype):
     """The fused row epilogues against the float64 row-by-row oracle (oracle/blocks.py) on the same (rounded) inputs:
     every pre / LayerNorm / post combination the blocks use, rows that do not fill a workgroup.
