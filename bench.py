@@ -182,10 +182,14 @@ def backward_section(torch, ops, steps, warmup):
         return median_us(torch, fn, steps, warmup)[0]
 
     us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
+    kh, vh, gyh = k.bfloat16(), v.bfloat16(), gy.bfloat16()
+    us_bh = timed(lambda: ops.bi_wkv_backward(w, u, kh, vh, gyh))
     us_6 = timed(lambda: ops.wkv6_backward(B, T, C, Hw, r6, k6, v6, w6, u6, gy))
     bytes_b = 5 * B * T * C * 4                                  # k, v, gy read; gk, gv written
     return {"biwkv_bwd_us_per_call": round(us_b, 2), "biwkv_bwd_GBps": round(bytes_b / (us_b * 1e-6) / 1e9, 1),
             "biwkv_bwd_pct_hbm_peak": round(100 * bytes_b / (us_b * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
+            "biwkv_bwd_bf16_us_per_call": round(us_bh, 2),
+            "biwkv_bwd_bf16_pct_hbm_peak": round(100 * bytes_b / 2 / (us_bh * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
             "wkv6_bwd_us_per_call": round(us_6, 1), "wkv6_bwd_tokens_per_s": round(B * T / (us_6 * 1e-6), 1)}
 
 
