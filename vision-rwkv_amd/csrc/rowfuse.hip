@@ -405,6 +405,10 @@ template <typename IO, int VPL, int W, int PRE, int POST>
 int launch_ln(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
               long long rows, int N, float eps, hipStream_t st) {
     constexpr int per_wg = (W == 1 ? 4 : 1) * rows_per_group_fwd<VPL>();
+    if ((rows + per_wg - 1) / per_wg > 0x7fffffffLL) {
+        set_error("rowfuse: too many rows (%lld)", rows);
+        return VRWKV_UNSUPPORTED_SHAPE;
+    }
     const dim3 block(256), grid((unsigned)((rows + per_wg - 1) / per_wg));
     const IO *pa = static_cast<const IO*>(a), *po = static_cast<const IO*>(other), *pw = static_cast<const IO*>(lnw),
              *pb = static_cast<const IO*>(lnb), *pg = static_cast<const IO*>(gamma);
