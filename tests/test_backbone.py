@@ -423,3 +423,43 @@ def test_vrwkv6_mix_backward_against_autograd(B, T, C, dtype):
             assert y.grad.dtype == ydt
             check("gy", y.grad, y2.grad); check("ggate", gate.grad, g2.grad)
             check("gw", w.grad, w2.grad); check("gb", b.grad, b2.grad)
+
+
+@pytest.mark.gpu
+def test_split_weight_gradient_of_the_block_projections():
+    """The bias-free projections of a block under autograd with many tokens (backbone._proj, backbone._matmul): the
+    weight gradient is a sum of batched partial products over the tokens; forward and input gradient are the plain
+    GEMMs (bit-identical), the weight gradient agrees with the float32 product as well as the library's own bf16 GEMM
+    does.  Few tokens, a bias or fp32 take the plain path."""
+    from vision_rwkv_amd import backbone as bb
+    dev = "cuda:0"
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(192, 320, bias=False).to(dev).bfloat16()
+    x = torch.randn(8, 1024, 192, device=dev).bfloat16().requires_grad_(True)
+    g = torch.randn(8, 1024, 320, device=dev).bfloat16()
+    y1 = bb._proj(lin, x)
+    assert y1.grad_fn is not None and "SplitKLinear" in type(y1.grad_fn).__name__
+    y1.backward(g)
+    gx1, gw1 = x.grad.clone(), lin.weight.grad.clone()
+    x.grad = None
+    lin.weight.grad = None
+    y2 = lin(x)
+    y2.backward(g)
+    assert torch.equal(y1, y2) and torch.equal(gx1, x.grad)
+    ref = g.float().reshape(-1, 320).t() @ x.detach().float().reshape(-1, 192)
+    scale = ref.abs().max()
+    err_split = ((gw1.float() - ref).abs().max() / scale).item()
+    err_plain = ((lin.weight.grad.float() - ref).abs().max() / scale).item()
+    assert err_split <= max(2 * err_plain, 4e-3), (err_split, err_plain)
+    w = (torch.randn(192, 40, device=dev) * 0.05).bfloat16().requires_grad_(True)
+    z = bb._matmul(x.detach(), w)
+    assert "SplitKMatmul" in type(z.grad_fn).__name__
+    gz = torch.randn_like(z)
+    z.backward(gz)
+    refw = x.detach().float().reshape(-1, 192).t() @ gz.float().reshape(-1, 40)
+    assert ((w.grad.float() - refw).abs().max() / refw.abs().max()).item() <= 4e-3
+    # plain paths
+    small = torch.randn(2, 16, 192, device=dev).bfloat16().requires_grad_(True)
+    assert "SplitK" not in type(bb._proj(lin, small).grad_fn).__name__
+    with torch.no_grad():
+        assert bb._proj(lin, x).grad_fn is None

@@ -58,6 +58,77 @@ def _mix(module, x, mixes, shift_pixel, gamma, patch_resolution, fused, head_dim
     return [x * m + xx * (1 - m) for m in mixes]
 
 
+class _SplitKLinear(torch.autograd.Function):
+    """x @ W^T whose weight gradient g^T x -- a contraction over all B*T tokens into a small (out, in) matrix, which the
+    library's GEMM runs as one deep sum on too few workgroups -- is computed as `splits` batched partial products that
+    are added in fp32.  Forward and input gradient are the library's plain GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, weight, splits):
+        ctx.save_for_backward(x, weight)
+        ctx.splits = splits
+        return F.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        S = ctx.splits
+        gx = g @ weight if ctx.needs_input_grad[0] else None
+        gw = None
+        if ctx.needs_input_grad[1]:
+            g2, x2 = g.reshape(-1, g.shape[-1]), x.reshape(-1, x.shape[-1])
+            M = g2.shape[0]
+            part = torch.bmm(g2.view(S, M // S, -1).transpose(1, 2), x2.view(S, M // S, -1))
+            gw = part.sum(0, dtype=torch.float32).to(weight.dtype)    # partial products added in fp32
+        return gx, gw, None
+
+
+class _SplitKMatmul(torch.autograd.Function):
+    """x @ W for a parameter matrix W (in, out): the same split of the weight gradient x^T g over the tokens."""
+
+    @staticmethod
+    def forward(ctx, x, weight, splits):
+        ctx.save_for_backward(x, weight)
+        ctx.splits = splits
+        return x @ weight
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        S = ctx.splits
+        gx = g @ weight.t() if ctx.needs_input_grad[0] else None
+        gw = None
+        if ctx.needs_input_grad[1]:
+            g2, x2 = g.reshape(-1, g.shape[-1]), x.reshape(-1, x.shape[-1])
+            M = g2.shape[0]
+            part = torch.bmm(x2.view(S, M // S, -1).transpose(1, 2), g2.view(S, M // S, -1))
+            gw = part.sum(0, dtype=torch.float32).to(weight.dtype)    # partial products added in fp32
+        return gx, gw, None
+
+
+def _matmul(x, weight):
+    """x @ weight for a low-rank parameter matrix; split weight gradient under autograd with many tokens."""
+    if (x.is_cuda and torch.is_grad_enabled() and weight.requires_grad and x.dtype == weight.dtype
+            and x.dtype in (torch.bfloat16, torch.float16) and weight.dim() == 2):
+        M = x.numel() // x.shape[-1]
+        if M >= 4096 and M % 8 == 0:
+            return _SplitKMatmul.apply(x, weight, 8)
+    return x @ weight
+
+
+def _proj(linear, x):
+    """linear(x) for the bias-free projections of a block; under autograd on the GPU with many tokens the weight gradient
+    is split over the tokens (see _SplitKLinear)."""
+    w = linear.weight
+    if (linear.bias is None and x.is_cuda and torch.is_grad_enabled() and w.requires_grad and x.dtype == w.dtype
+            and x.dtype in (torch.bfloat16, torch.float16)):
+        M = x.numel() // x.shape[-1]
+        S = 4 if w.numel() >= (1 << 21) else 8
+        if M >= 4096 and M % S == 0:
+            return _SplitKLinear.apply(x, w, S)
+    return linear(x)
+
+
 def _layer_norm(ln, x):
     """nn.LayerNorm over the channels through the fused row kernel (forward and backward); tensor ops where it does
     not apply."""
@@ -92,7 +163,7 @@ class VRWKV_SpatialMix(nn.Module):
                               self.channel_gamma, patch_resolution, self.fused_shift)
         else:
             xk = xv = xr = x
-        k, v, r = self.key(xk), self.value(xv), self.receptance(xr)
+        k, v, r = _proj(self.key, xk), _proj(self.value, xv), _proj(self.receptance, xr)
         wd = self.spatial_decay.dtype
         if torch.is_grad_enabled() or k.dtype != (wd if wd in (torch.half, torch.bfloat16) else torch.float32):
             y = RUN_CUDA(self.spatial_decay / T, self.spatial_first / T, k, v)  # vrwkv.py:183
@@ -107,7 +178,7 @@ class VRWKV_SpatialMix(nn.Module):
         kn = self.key_norm
         y = row_fuse(y, r, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
                      PRE_NONE, POST_SIGMOID_GATE, kn.eps if kn is not None else 1e-5)
-        return self.output(y)
+        return _proj(self.output, y)
 
 
 class VRWKV_ChannelMix(nn.Module):
@@ -133,9 +204,9 @@ class VRWKV_ChannelMix(nn.Module):
             xk = xr = x
         # relu^2 (+ key_norm) and the sigmoid gate (vrwkv.py:256-261), one pass each; tensor ops under autograd
         kn = self.key_norm
-        k = row_fuse(self.key(xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
+        k = row_fuse(_proj(self.key, xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
                      PRE_RELU_SQ, POST_NONE, kn.eps if kn is not None else 1e-5)
-        return row_fuse(self.value(k), self.receptance(xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
+        return row_fuse(_proj(self.value, k), _proj(self.receptance, xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
 
 
 class Block(nn.Module):

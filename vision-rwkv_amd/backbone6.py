@@ -10,7 +10,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .backbone import VRWKV, eval_cached
+from .backbone import VRWKV, eval_cached, _proj, _matmul
 from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, q_shift_mix_autograd, stack_mixes, row_fuse, maa_mix, groupnorm_gate, PRE_NONE, PRE_RELU_SQ, POST_NONE,
                   POST_SIGMOID_GATE, POST_RESIDUAL)
 
@@ -85,7 +85,7 @@ class VRWKV_SpatialMix_V6(nn.Module):
         sx, xxx = _shift_and_mix(self, x, lambda: [torch.zeros_like(self.time_maa_x), 1 - self.time_maa_x],
                                  self.shift_pixel, patch_resolution, self.with_cls_token, self.fused_shift,
                                  (self.time_maa_x,))
-        lo = torch.tanh(xxx @ self.time_maa_w1).view(B * T, 5, -1).transpose(0, 1)
+        lo = torch.tanh(_matmul(xxx, self.time_maa_w1)).view(B * T, 5, -1).transpose(0, 1)
         m = torch.bmm(lo, self.time_maa_w2).view(5, B, T, C)
         # xw..xg = x + (sx - x) * (time_maa_* + m_*)  (vrwkv6.py:190-194): one pass at inference
         maas = (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g)
@@ -93,9 +93,9 @@ class VRWKV_SpatialMix_V6(nn.Module):
         if not torch.is_grad_enabled() and x.is_cuda:
             table = eval_cached(self, "maa_table", maas, x.device, lambda: stack_mixes(maas, x.device))
         xw, xk, xv, xr, xg = maa_mix(x, sx, m, maas, table)
-        r, k, v = self.receptance(xr), self.key(xk), self.value(xv)
-        gate = self.gate(xg)
-        w = self.time_decay + torch.tanh(xw @ self.time_decay_w1) @ self.time_decay_w2
+        r, k, v = _proj(self.receptance, xr), _proj(self.key, xk), _proj(self.value, xv)
+        gate = _proj(self.gate, xg)
+        w = self.time_decay + _matmul(torch.tanh(_matmul(xw, self.time_decay_w1)), self.time_decay_w2)
         y = RUN_CUDA_RWKV6(B, T, C, self.n_head, r.contiguous(), k.contiguous(), v.contiguous(),
                            w.contiguous(), self.time_faaaa.float())                  # vrwkv6.py:217 (w as it is: the
         # kernel widens a 16-bit decay logit itself, the same values the reference's `w.float()` holds)
@@ -103,7 +103,7 @@ class VRWKV_SpatialMix_V6(nn.Module):
             y = self.key_norm(y.to(gate.dtype))
         # ln_x over each head's channels, times silu(gate) (vrwkv6.py:199, 205-211): one pass at inference
         y = groupnorm_gate(y, gate, self.ln_x.weight, self.ln_x.bias, self.ln_x.num_groups, self.ln_x.eps)
-        return self.output(y)
+        return _proj(self.output, y)
 
 
 class VRWKV_ChannelMix_V6(nn.Module):
@@ -127,9 +127,9 @@ class VRWKV_ChannelMix_V6(nn.Module):
                                 patch_resolution, self.with_cls_token, self.fused_shift,
                                 (self.spatial_mix_k, self.spatial_mix_r))
         kn = self.key_norm                                   # relu^2 (+ key_norm), then the sigmoid gate: one pass each
-        k = row_fuse(self.key(xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
+        k = row_fuse(_proj(self.key, xk), None, kn.weight if kn is not None else None, kn.bias if kn is not None else None, None,
                      PRE_RELU_SQ, POST_NONE, kn.eps if kn is not None else 1e-5)
-        return row_fuse(self.value(k), self.receptance(xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
+        return row_fuse(_proj(self.value, k), _proj(self.receptance, xr), None, None, None, PRE_NONE, POST_SIGMOID_GATE)
 
 
 class Block6(nn.Module):
