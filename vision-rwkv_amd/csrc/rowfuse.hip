@@ -7,8 +7,9 @@
 //   :256-260  k = square(relu(key(xk))); k = key_norm(k)           -> a = key(xk), pre = relu^2, LayerNorm
 //   :261      sigmoid(receptance(xr)) * kv                         -> a = kv, other = receptance(xr), sigmoid gate
 //   :300-313  x = x + gamma * ln(att(x)) / x + gamma * att(ln(x))  -> a = branch output, other = x, (LayerNorm,) gamma
-// One wave per row: a lane keeps its 16-byte vectors of the row in registers (read once), the mean and the variance are
-// reduced across the wave in fp32 (two passes over the registers), the result is written once.
+// One wave per row of up to 128 16-byte vectors, the four waves of a workgroup per longer row: a thread keeps its vectors
+// of the row in registers (read once, every load of a group's rows issued before the first value is used), the mean and
+// the variance are reduced in fp32 (two passes over the registers), the result is written once.
 //
 // Backward (vrwkv_rowfuse_bwd; the reference differentiates the PyTorch ops by autograd): with g the gradient of out,
 // z = pre(a), xh = (z - mean) rstd, y = xh w + b (y = z without LayerNorm):
