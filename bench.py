@@ -222,7 +222,7 @@ def sweep_section(torch, ops, steps, warmup):
     return rows
 
 
-def elementwise_section(torch, ops):
+def elementwise_section(torch, ops, which="b,l"):
     """The element-wise kernels of a block (q_shift + mixes, the row-wise epilogues, the VRWKV6 mix steps) at the
     VRWKV-B layer shape (64, 196, 768) and the VRWKV-L one (32, 576, 1024), bf16: each timed as calls on rotating
     buffer sets back to back (six sets, more than the last-level cache holds), in us and GB/s of the algorithmic
@@ -254,7 +254,8 @@ def elementwise_section(torch, ops):
         return sorted(r)[len(r) // 2]
 
     out = []
-    for (Bn, Hp, Wp, Cn) in ((64, 14, 14, 768), (32, 24, 24, 1024)):
+    shapes = {"b": (64, 14, 14, 768), "l": (32, 24, 24, 1024)}
+    for (Bn, Hp, Wp, Cn) in [shapes[k] for k in which.split(",") if k in shapes]:
         Tn = Hp * Wp
         n = Bn * Tn * Cn
         g = torch.Generator(device="cpu").manual_seed(Cn)
@@ -449,6 +450,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the dense-prediction shape sweep (B=2, long T)")
     ap.add_argument("--no-config2", action="store_true", help="skip the B=2, T=4150, C=768 bf16 measurement")
     ap.add_argument("--no-elementwise", action="store_true", help="skip the element-wise block kernels (q_shift + mix, row epilogues)")
+    ap.add_argument("--elementwise-shapes", default="b,l",
+                    help="layer shapes of the element-wise section: b = (64, 196, 768), l = (32, 576, 1024)")
     ap.add_argument("--cpu-calls", type=int, default=96)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of a (B,T,C) fp32 tensor (a kernel of known "
@@ -582,7 +585,7 @@ def main():
     if not args.no_sweep:
         out["sweep"] = sweep_section(torch, ops, 10, 3)
     if not args.no_elementwise:
-        out["elementwise"] = elementwise_section(torch, ops)
+        out["elementwise"] = elementwise_section(torch, ops, args.elementwise_shapes)
     if not args.no_backbone:
         out["backbone"] = backbone_section(torch, ops, 5, 3)
     print(json.dumps(out))
