@@ -120,8 +120,9 @@ def _proj(linear, x):
     """linear(x) for the bias-free projections of a block; under autograd on the GPU with many tokens the weight gradient
     is split over the tokens (see _SplitKLinear)."""
     w = linear.weight
-    if (linear.bias is None and x.is_cuda and torch.is_grad_enabled() and w.requires_grad and x.dtype == w.dtype
-            and x.dtype in (torch.bfloat16, torch.float16)):
+    hooked = linear._forward_hooks or linear._forward_pre_hooks       # hooks fire only through linear(x)
+    if (linear.bias is None and not hooked and x.is_cuda and torch.is_grad_enabled() and w.requires_grad
+            and x.dtype == w.dtype and x.dtype in (torch.bfloat16, torch.float16)):
         M = x.numel() // x.shape[-1]
         S = 4 if w.numel() >= (1 << 21) else 8
         if M >= 4096 and M % S == 0:
@@ -241,12 +242,21 @@ class Block(nn.Module):
 
 
 class VRWKV(nn.Module):
-    """vrwkv.py:322-432 without the mmcv base classes; returns the last feature map (B, C, Hp, Wp)."""
+    """vrwkv.py:322-432 without the mmcv base classes.  With `out_indices` left at None it returns the last feature map
+    (B, C, Hp, Wp); with an int or a sequence of layer indices (negative ones count from the end) it returns the tuple
+    of those layers' feature maps, as the reference does for the mmdet / mmseg callers (vrwkv.py:368-378, 421-432)."""
 
     def __init__(self, img_size=224, patch_size=16, in_channels=3, embed_dims=256, depth=12, channel_gamma=1 / 4,
                  shift_pixel=1, post_norm=False, key_norm=False, init_values=None, hidden_rate=4, final_norm=True,
-                 interpolate_mode="bicubic", fused_shift=True):
+                 interpolate_mode="bicubic", fused_shift=True, out_indices=None):
         super().__init__()
+        if out_indices is not None:
+            out_indices = [out_indices] if isinstance(out_indices, int) else list(out_indices)
+            out_indices = [depth + i if i < 0 else i for i in out_indices]
+            for i in out_indices:
+                if not 0 <= i <= depth:
+                    raise ValueError(f"Invalid out_indices {i}")
+        self.out_indices = out_indices
         self.patch_size = patch_size
         self.patch_embed = nn.Conv2d(in_channels, embed_dims, kernel_size=patch_size, stride=patch_size, bias=True)
         self.patch_resolution = (img_size // patch_size, img_size // patch_size)
@@ -313,11 +323,17 @@ class VRWKV(nn.Module):
     def forward(self, img):
         x, res = self.embed(img)
         x = x + self._pos_embed_for(res).to(x.dtype)
-        for layer in self.layers:
-            x = layer(x, res)
-        if self.final_norm:
-            x = _layer_norm(self.ln1, x)
         B, _, C = x.shape
+        outs = []
+        last = len(self.layers) - 1
+        for i, layer in enumerate(self.layers):
+            x = layer(x, res)
+            if i == last and self.final_norm:
+                x = _layer_norm(self.ln1, x)
+            if self.out_indices is not None and i in self.out_indices:
+                outs.append(x.reshape(B, res[0], res[1], C).permute(0, 3, 1, 2))
+        if self.out_indices is not None:
+            return tuple(outs)
         return x.reshape(B, res[0], res[1], C).permute(0, 3, 1, 2)
 
 
