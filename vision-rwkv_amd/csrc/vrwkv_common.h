@@ -155,19 +155,23 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 }
 // ---- per-phase cycle stamps (instrumented build only: -DVRWKV_STAMPS, `make stamps`) ----------------------------
 // A wave records the shader clock at numbered points of a tile into a buffer the host registered with
-// vrwkv_debug_set_stamp_buffer: layout [workgroup][wave (8)][tile slot (VRWKV_STAMP_TILES)][point (VRWKV_STAMP_POINTS)].
+// vrwkv_debug_set_stamp_buffer_<tag>(buffer, n_workgroups): layout [workgroup][wave (8)][tile slot (VRWKV_STAMP_TILES)]
+// [point (VRWKV_STAMP_POINTS)]; workgroups beyond the count the buffer was sized for record nothing.
 #ifdef VRWKV_STAMPS
 constexpr int VRWKV_STAMP_TILES = 4, VRWKV_STAMP_POINTS = 12;
 static __device__ unsigned long long* g_stamp_buffer = nullptr;   // one per translation unit (device code is not linked across them)
-// defines vrwkv_debug_set_stamp_buffer_<tag>(device_buffer) for the translation unit it is used in
+static __device__ unsigned g_stamp_workgroups = 0;                // workgroups the buffer has room for
+// defines vrwkv_debug_set_stamp_buffer_<tag>(device_buffer, n_workgroups) for the translation unit it is used in
 #define VRWKV_DEFINE_STAMP_SETTER(tag)                                                                      \
-    extern "C" int vrwkv_debug_set_stamp_buffer_##tag(void* device_buffer) {                                 \
+    extern "C" int vrwkv_debug_set_stamp_buffer_##tag(void* device_buffer, unsigned n_workgroups) {          \
         unsigned long long* p = static_cast<unsigned long long*>(device_buffer);                             \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(::vrwkv::g_stamp_workgroups), &n_workgroups, sizeof(n_workgroups)) != hipSuccess) return 4; \
         return hipMemcpyToSymbol(HIP_SYMBOL(::vrwkv::g_stamp_buffer), &p, sizeof(p)) == hipSuccess ? 0 : 4;   \
     }
 __device__ __forceinline__ void stamp(int wave, int slot, int point) {
     unsigned long long* buf = g_stamp_buffer;
-    if (buf && slot < VRWKV_STAMP_TILES && (threadIdx.x & 63) == 0) {
+    if (buf && blockIdx.x < g_stamp_workgroups && wave < 8 && slot < VRWKV_STAMP_TILES && point < VRWKV_STAMP_POINTS &&
+        (threadIdx.x & 63) == 0) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         buf[(((size_t)blockIdx.x * 8 + wave) * VRWKV_STAMP_TILES + slot) * VRWKV_STAMP_POINTS + point] = __builtin_amdgcn_s_memtime();
     }
