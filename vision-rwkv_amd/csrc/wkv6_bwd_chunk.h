@@ -30,7 +30,7 @@
 // clears its sequence's flag on entry and a scan only ever sets one, so a sequence that any of the six scans gave
 // up on is redone.
 #pragma once
-#include "wkv6_fwd_chunk.h"
+#include "wkv6_chunk_common.h"
 
 namespace vrwkv {
 namespace wkv6_detail {

@@ -57,15 +57,15 @@ int launch_scalar(const void* r, const void* k, const void* v, const void* w, co
 template <typename IO, typename WT>
 int launch_chunked(const void* r, const void* k, const void* v, const void* w, const float* u, float* y,
                    int B, int T, int C, int H, bool w_is_ew, hipStream_t st) {
-    const dim3 grid(B * H), block(256);
+    const dim3 grid(B * H), block(64 * FW_WAVES);
     const IO* rr = static_cast<const IO*>(r);
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
     const WT* ww = static_cast<const WT*>(w);
     if (w_is_ew)
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, true>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H, nullptr);
     else
-        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H);
+        hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<IO, WT, false>), grid, block, 0, st, rr, kk, vv, ww, u, y, T, C, H, nullptr);
     return check_launch("wkv6_fwd (chunked)");
 }
 
@@ -80,6 +80,37 @@ int launch_any(const void* r, const void* k, const void* v, const void* w, const
 }
 
 }  // namespace
+
+extern "C" size_t vrwkv_wkv6_fwd_phases_bytes(int B, int T, int H) {
+    if (B <= 0 || T <= 0 || H <= 0) return 0;
+    return (size_t)B * H * FW_WAVES * ((T + LC - 1) / LC) * FW_STAMP_POINTS * sizeof(unsigned long long);
+}
+
+extern "C" int vrwkv_wkv6_fwd_phases(const void* r, const void* k, const void* v, const void* w, const float* u,
+                                     float* y, int B, int T, int C, int H, void* stamps, size_t stamp_bytes,
+                                     void* hip_stream) {
+    int rc = validate(B, T, C, H, VRWKV_BF16, VRWKV_F32);
+    if (rc != VRWKV_OK) return rc;
+    if (!r || !k || !v || !w || !u || !y || !stamps) {
+        set_error("wkv6_fwd_phases: null pointer argument");
+        return VRWKV_INVALID_ARG;
+    }
+    if ((((uintptr_t)r | (uintptr_t)k | (uintptr_t)v) & 1) || (((uintptr_t)w | (uintptr_t)u | (uintptr_t)y) & 3) ||
+        ((uintptr_t)stamps & 7)) {
+        set_error("wkv6_fwd_phases: pointers must be aligned to their element size");
+        return VRWKV_INVALID_ARG;
+    }
+    const size_t need = vrwkv_wkv6_fwd_phases_bytes(B, T, H);
+    if (stamp_bytes < need) {
+        set_error("wkv6_fwd_phases: stamp buffer of %zu bytes required (got %zu)", need, stamp_bytes);
+        return VRWKV_WORKSPACE_TOO_SMALL;
+    }
+    hipLaunchKernelGGL((wkv6_fwd_chunk_kernel<__hip_bfloat16, float, false, true>), dim3(B * H), dim3(64 * FW_WAVES), 0,
+                       static_cast<hipStream_t>(hip_stream), static_cast<const __hip_bfloat16*>(r),
+                       static_cast<const __hip_bfloat16*>(k), static_cast<const __hip_bfloat16*>(v),
+                       static_cast<const float*>(w), u, y, T, C, H, static_cast<unsigned long long*>(stamps));
+    return check_launch("wkv6_fwd_phases");
+}
 
 extern "C" size_t vrwkv_wkv6_fwd_workspace_bytes(int B, int T, int C, int H) {
     (void)B; (void)T; (void)C; (void)H;
