@@ -84,7 +84,7 @@ template <bool VSPLIT>
 struct __attribute__((aligned(16))) FwdLds {
     __bf16 Rh[LC][FW_PJ], Rl[LC][FW_PJ], Kh[LC][FW_PJ], Kl[LC][FW_PJ];
     __bf16 Kth[HN][FW_PS], Ktl[HN][FW_PS], Vt[HN][FW_PS], Vtl[VSPLIT ? HN : 1][FW_PS];
-    float C2[HN], Tot[4][HN], Bon[4][LC];
+    float C2[4][HN], Tot[4][HN], Bon[4][LC];     // C2: e^P31 per channel, one copy per wave (written and read by that wave only)
 };
 
 // Phase stamps (STAMPS = true, the profiling entry point only): lane 0 of every wave stores the shader clock at
@@ -229,6 +229,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
     fetch_rkv(0, C);
     decay_sums(0, C, p);
     f32x4v accY[2];                                                      // y tiles of the step: filled in E (earlier values), finished in M
+    bf16x8 zh[2], zl[2];                                                 // the scaled state of the step as MFMA operands (formed in E)
     unsigned y_lane = 0;
     sync_step();
 
@@ -250,6 +251,10 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // ascending one in half 2 cy + 1; this step's E runs in half hp, its M in half hp + 1
         const int other_m = asc ? 2 * (nchunk - cy) : 2 * cy + 1;
         const bool y_second = other_m < hp + 1, y_late = other_m == hp;   // wave-uniform
+        // ... and if the other pass runs its E of chunk cy in the half of this step's M, it fetches this step's y rows
+        // right behind the barrier that ends that half: then the stores are waited for before that barrier (the barrier
+        // orders the instructions' issue, not the arrival of the data)
+        const bool y_drain = (asc ? 2 * (nchunk - 1 - cy) + 1 : 2 * cy) == hp + 1;
         {
             // =============================== stage E: elementwise =================================
             // wave w4 of the pass prepares tokens n = 8 w4 .. 8 w4 + 7 of the chunk; lane = channel j (and i for v)
@@ -259,14 +264,32 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             // operand is one 16-byte read: j = 32 kb + 16 hf + 4 g + e  ->  column 32 kb + 8 g + 4 hf + e.
             const int jcol = (lane_e & 32) | ((lane_e & 12) << 1) | ((lane_e & 16) >> 2) | (lane_e & 3);
             stamp(ch, 0);
-            // rest = log2 decay from the start of this wave's tokens to the chunk's end; P_m - P31 = p[m] - rest >= 0
-            float rest = L.Tot[3][lane_e];
-            if (w4 <= 2) rest += L.Tot[2][lane_e];
-            if (w4 <= 1) rest += L.Tot[1][lane_e];
-            if (w4 == 0) {
-                rest += L.Tot[0][lane_e];                                // = P31 (log2 units)
-                L.C2[lane_e] = fast_exp2(rest);
-                if (__builtin_amdgcn_ballot_w64(!(rest >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag[hp & 1] = 1;
+            // The next chunk's decay rows: summed at the end of this step's matrix stage, a whole step of latency away (the
+            // last step re-reads its own rows: no branch, so the compiler's wait counts stay exact).
+            fetch_w(ch + 1 < nchunk ? ch + 1 : ch, Cs);
+            // rest = log2 decay from the start of this wave's tokens to the chunk's end (P_m - P31 = p[m] - rest >= 0),
+            // p31 = that of the whole chunk; the waves' totals were written at the end of the previous matrix stage
+            const float t0 = L.Tot[0][lane_e], t1 = L.Tot[1][lane_e], t2 = L.Tot[2][lane_e], t3 = L.Tot[3][lane_e];
+            const float m0 = w4 == 0 ? 1.f : 0.f, m1 = w4 <= 1 ? 1.f : 0.f, m2 = w4 <= 2 ? 1.f : 0.f;     // wave-uniform
+            const float rest = fmaf(m0, t0, fmaf(m1, t1, fmaf(m2, t2, t3)));
+            const float p31 = (t0 + t1) + (t2 + t3);
+            if (w4 == 0 && __builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag[hp & 1] = 1;
+            // Z = diag(e^P31) S, in place, split into head and tail for MFMA 3 (done here, while the r, k, v rows are still
+            // on their way): a lane needs e^P31 of the channels its state rows belong to, taken from the wave's own copy
+            L.C2[w4][lane_e] = fast_exp2(p31);
+            {
+                const int g4 = lane_e >> 4;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    float z8[8];
+#pragma unroll
+                    for (int hf = 0; hf < 2; ++hf) {
+                        const f32x4 c2 = *reinterpret_cast<const f32x4*>(&L.C2[w4][16 * (2 * kb + hf) + 4 * g4]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { S[2 * kb + hf][e] *= c2[e]; z8[4 * hf + e] = S[2 * kb + hf][e]; }
+                    }
+                    split8(z8, zh[kb], zl[kb]);
+                }
             }
             {
                 unsigned kthw[4], ktlw[4], vthw[4], vtlw[4];
@@ -329,8 +352,6 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             // ================================= stage M: matrix cores ===============================
             const int g4 = lane_e >> 4, c16 = lane_e & 15;                // lane = (column c16, slot group g4)
             stamp(ch, 4);
-            fetch_w(ch + 1 < nchunk ? ch + 1 : ch, Cs);    // next chunk's decays, summed at the end of this stage (no branch:
-                                                           // the compiler's wait counts stay exact; the last step re-reads its own)
             if (y_late) {
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb) accY[tb] = __builtin_bit_cast(f32x4v, BufRaw<16>::ld(rsy, y_lane, y_row(cy, tb, Cs)));
@@ -345,15 +366,11 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 return *reinterpret_cast<const bf16x8*>(&arr[16 * blk + c16][32 * kb + 8 * g4]);
             };
             f32x4v accA[3] = {f32x4v{0.f, 0.f, 0.f, 0.f}, f32x4v{0.f, 0.f, 0.f, 0.f}, f32x4v{0.f, 0.f, 0.f, 0.f}};
-            bf16x8 zh[2], zl[2];
-    #pragma unroll
+#pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 // ---- phase kb: operands of contraction half kb ----
                 bf16x8 RH[2], RL[2], KH[2], KL[2];
-                f32x4 c2[2];
-    #pragma unroll
-                for (int hf = 0; hf < 2; ++hf) c2[hf] = *reinterpret_cast<const f32x4*>(&L.C2[16 * (2 * kb + hf) + 4 * g4]);
-    #pragma unroll
+#pragma unroll
                 for (int blk = 0; blk < 2; ++blk) {
                     RH[blk] = rows_op(L.Rh, blk, kb);
                     RL[blk] = rows_op(L.Rl, blk, kb);
@@ -361,32 +378,23 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     KL[blk] = rows_op(L.Kl, blk, kb);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                // Z = diag(e^P31) S, in place, split into head and tail
-                {
-                    float z8[8];
-    #pragma unroll
-                    for (int hf = 0; hf < 2; ++hf)
-    #pragma unroll
-                        for (int e = 0; e < 4; ++e) { S[2 * kb + hf][e] *= c2[hf][e]; z8[4 * hf + e] = S[2 * kb + hf][e]; }
-                    split8(z8, zh[kb], zl[kb]);
-                }
                 // MFMA 3: Y^T += Z^T rt^T with Z straight from the accumulators (the state tile is the A operand: rows = value
             // columns, so the y tiles come out transposed);
                 // MFMA 1: A^T blocks (s block, t block) = (0,0), (0,1), (1,1): acc[m = s][n = t]; the lane holds t = c16 of the
                 // block, rows s = 4 g4 + r.  Block (1,0) has s > t throughout.
-    #pragma unroll
+#pragma unroll
                 for (int tb = 0; tb < 2; ++tb) {
                     accY[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zh[kb], RH[tb], accY[tb], 0, 0, 0);
                     accA[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KH[0], RH[tb], accA[tb], 0, 0, 0);
                 }
                 accA[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KH[1], RH[1], accA[2], 0, 0, 0);
-    #pragma unroll
+#pragma unroll
                 for (int tb = 0; tb < 2; ++tb) {
                     accY[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zl[kb], RH[tb], accY[tb], 0, 0, 0);
                     accA[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KH[0], RL[tb], accA[tb], 0, 0, 0);
                 }
                 accA[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KH[1], RL[1], accA[2], 0, 0, 0);
-    #pragma unroll
+#pragma unroll
                 for (int tb = 0; tb < 2; ++tb) {
                     accY[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zh[kb], RL[tb], accY[tb], 0, 0, 0);
                     accA[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KL[0], RH[tb], accA[tb], 0, 0, 0);
@@ -405,10 +413,10 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 bsl = *reinterpret_cast<const bf16x8*>(&L.Vtl[icol][8 * g4]);
             }
             bf16x8 kth[4], ktl[4];
-    #pragma unroll
+#pragma unroll
             for (int jt = 0; jt < 4; ++jt) kth[jt] = *reinterpret_cast<const bf16x8*>(&L.Kth[16 * jt + c16][8 * g4]);
             float bon[2];
-    #pragma unroll
+#pragma unroll
             for (int tb = 0; tb < 2; ++tb) {
                 const int t = 16 * tb + c16;
                 bon[tb] = (L.Bon[0][t] + L.Bon[1][t]) + (L.Bon[2][t] + L.Bon[3][t]);
@@ -421,24 +429,24 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             unsigned keepw[2], diagw[2];
             {
                 const int d = c16 - 4 * g4;                                   // t - s of register 0
-    #pragma unroll
+#pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     keepw[pr] = (2 * pr < d ? 0xffffu : 0u) | (2 * pr + 1 < d ? 0xffff0000u : 0u);
                     diagw[pr] = (2 * pr == d ? 0xffffu : 0u) | (2 * pr + 1 == d ? 0xffff0000u : 0u);
                 }
             }
             unsigned ahw[3][2], alw[3][2];
-    #pragma unroll
+#pragma unroll
             for (int blk = 0; blk < 3; ++blk) {
                 const float a4[4] = {accA[blk][0], accA[blk][1], accA[blk][2], accA[blk][3]};
                 split4(a4, ahw[blk], alw[blk]);
             }
-    #pragma unroll
+#pragma unroll
             for (int tb = 0; tb < 2; ++tb) {
                 const int blk = 2 * tb;
                 const float diag = asc ? bon[tb] : 0.f;
                 const unsigned dgh = pack_bf16(diag, diag), dgl = pack_bf16(diag - bf16_lo(dgh), diag - bf16_lo(dgh));
-    #pragma unroll
+#pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     ahw[blk][pr] = (ahw[blk][pr] & keepw[pr]) | (dgh & diagw[pr]);
                     alw[blk][pr] = (alw[blk][pr] & keepw[pr]) | (dgl & diagw[pr]);
@@ -451,19 +459,19 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 const bf16x8 Ah0 = words8(ahw[0][0], ahw[0][1], 0u, 0u), Al0 = words8(alw[0][0], alw[0][1], 0u, 0u);
                 const bf16x8 Ah1 = words8(ahw[1][0], ahw[1][1], ahw[2][0], ahw[2][1]), Al1 = words8(alw[1][0], alw[1][1], alw[2][0], alw[2][1]);
                 // the tails of kt^T are read behind the first MFMAs of this phase (their registers were A's accumulators)
-    #pragma unroll
+#pragma unroll
                 for (int jt = 0; jt < 4; ++jt) ktl[jt] = *reinterpret_cast<const bf16x8*>(&L.Ktl[16 * jt + c16][8 * g4]);
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kth[jt], bs, S[jt], 0, 0, 0);
                 accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Ah0, accY[0], 0, 0, 0);
                 accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Ah1, accY[1], 0, 0, 0);
-    #pragma unroll
+#pragma unroll
                 for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ktl[jt], bs, S[jt], 0, 0, 0);
                 accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al0, accY[0], 0, 0, 0);
                 accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al1, accY[1], 0, 0, 0);
                 if constexpr (VSPLIT) {
-    #pragma unroll
+#pragma unroll
                     for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kth[jt], bsl, S[jt], 0, 0, 0);
                     accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bvl, Ah0, accY[0], 0, 0, 0);
                     accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bvl, Ah1, accY[1], 0, 0, 0);
@@ -478,6 +486,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 BufRaw<16>::st(__builtin_bit_cast(typename BufRaw<16>::type, accY[tb]), rsy, y_lane, y_row(cy, tb, Cs));
             // the next chunk's decay sums (its rows were fetched at the top of this stage)
             decay_sums(ch + 1 < nchunk ? ch + 1 : ch, Cs, p);
+            if (y_drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             stamp(ch, 5);
         }
         sync_step();
