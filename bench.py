@@ -55,6 +55,23 @@ def median_us(torch, fn, steps, warmup, calls_per_step=1, stream=None):
     return sorted(reps)[len(reps) // 2], reps
 
 
+CACHE_BYTES = 256 << 20       # last-level cache: buffer sets rotated in a timed loop add up to more than this
+
+
+def rotating(make_set, set_bytes, call, min_sets=6, max_sets=48):
+    """fn() that runs `call(*sets[i])` on the next of n pre-generated input sets each time it is invoked, with n chosen
+    so that the sets together exceed the last-level cache (no call finds its inputs cache-resident)."""
+    n = max(min_sets, min(max_sets, -(-int(1.25 * CACHE_BYTES) // max(1, set_bytes))))
+    sets = [make_set(i) for i in range(n)]
+    state = {"i": 0}
+
+    def fn():
+        a = sets[state["i"]]
+        state["i"] = (state["i"] + 1) % n
+        return call(*a)
+    return fn, sets
+
+
 def error_report(y, ref):
     """The two error measures of the parity tests, for one output against the float64 oracle."""
     import numpy as np
@@ -75,18 +92,23 @@ def config2_section(torch, ops, steps, warmup):
     Bn, Tn, Cn = 2, 4150, 768
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(2)
-    k = torch.randn(Bn, Tn, Cn, generator=g)
-    v = torch.randn(Bn, Tn, Cn, generator=g)
-    big = (torch.rand(Bn, Tn, 1, generator=g) < 0.01).float() * 7.0 + 1.0
-    k, v = (k * big).to(dev).bfloat16(), (v * big).to(dev).bfloat16()
+
+    def make(i):
+        k = torch.randn(Bn, Tn, Cn, generator=g)
+        v = torch.randn(Bn, Tn, Cn, generator=g)
+        big = (torch.rand(Bn, Tn, 1, generator=g) < 0.01).float() * 7.0 + 1.0
+        return (k * big).to(dev).bfloat16(), (v * big).to(dev).bfloat16()
     c = torch.arange(Cn, dtype=torch.float64)
     w = ((-5.0 + 8.0 * (c / (Cn - 1))) / Tn).float().to(dev)
     u = ((math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / Tn).float().to(dev)
-    us, reps = median_us(torch, lambda: ops.bi_wkv_forward(w, u, k, v), steps, warmup)
+    fn, sets = rotating(make, 2 * Bn * Tn * Cn * 2, lambda k, v: ops.bi_wkv_forward(w, u, k, v))
+    us, reps = median_us(torch, fn, steps, warmup)
+    k, v = sets[0]
     y = ops.bi_wkv_forward(w, u, k, v)
     ref = clib.biwkv_fwd(w.cpu().numpy(), u.cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy())
     byt = 3 * Bn * Tn * Cn * 2 + 2 * Cn * 4
-    return {"workload": f"Bi-WKV forward B={Bn} T={Tn} C={Cn}, bf16 I/O, fp32 state, 1% of tokens x8, one call per step",
+    return {"workload": f"Bi-WKV forward B={Bn} T={Tn} C={Cn}, bf16 I/O, fp32 state, 1% of tokens x8, one call per step, "
+                        f"{len(sets)} input sets in rotation",
             "us_per_call": round(us, 2), "repeats_us": [round(x, 2) for x in reps],
             "roofline": {"bound": "hbm", "achieved": round(byt / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(byt / us / 1e3 / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": byt,
@@ -126,15 +148,20 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
     Cw = Hw * 64
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(4321)
-    r, k, v = (torch.randn(Bw, Tw, Cw, generator=g).to(dev).bfloat16() for _ in range(3))
-    w = (torch.randn(Bw, Tw, Cw, generator=g) * 0.5 - 0.5).to(dev)
     u = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
-    us, reps = median_us(torch, lambda: ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u), steps, warmup)
+
+    def make(i):
+        r, k, v = (torch.randn(Bw, Tw, Cw, generator=g).to(dev).bfloat16() for _ in range(3))
+        return r, k, v, (torch.randn(Bw, Tw, Cw, generator=g) * 0.5 - 0.5).to(dev)
+    fn, sets = rotating(make, Bw * Tw * Cw * (3 * 2 + 4), lambda r, k, v, w: ops.wkv6_forward(Bw, Tw, Cw, Hw, r, k, v, w, u))
+    us, reps = median_us(torch, fn, steps, warmup)
+    r, k, v, w = sets[0]
     nchunk = (Tw + 31) // 32
-    # per chunk, pass and value half (one wave): 36 MFMA 32x32x16 = 36 * 32768 flop
-    mfma_flops = Bw * Hw * 2 * nchunk * 2 * 36 * 32768
+    # per chunk step a workgroup of eight waves issues 42 MFMA 16x16x32 per wave, 16384 flop each
+    waves, mfma_per_wave_step, mfma_flop, mfma_cycles = 8, 42, 2 * 16 * 16 * 32, 16
+    mfma_flops = Bw * Hw * nchunk * waves * mfma_per_wave_step * mfma_flop
     out = {
-        "workload": f"wkv6 forward B={Bw} T={Tw} C={Cw} H={Hw}, bf16 r,k,v, fp32 w,y",
+        "workload": f"wkv6 forward B={Bw} T={Tw} C={Cw} H={Hw}, bf16 r,k,v, fp32 w,y, {len(sets)} input sets in rotation",
         "us_per_call": round(us, 2),
         "repeats_us": [round(x, 2) for x in reps],
         "tokens_per_s": round(Bw * Tw / (us * 1e-6), 1),
@@ -142,6 +169,44 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
         "mfma_issued_tflops": round(mfma_flops / (us * 1e-6) / 1e12, 2),
         "pct_bf16_mfma_peak_end_to_end": round(100.0 * mfma_flops / (us * 1e-6) / 2.5e15, 3),
     }
+    # Matrix-pipe share inside the contraction stage: the library's profiling entry runs the same kernel with the shader
+    # clock stamped by every wave on entering and leaving the matrix stage of every chunk step; a wave's 42 MFMAs occupy
+    # the pipe for 16 cycles each (measured: a chain of dependent v_mfma_f32_16x16x32_bf16 issues one per 16 cycles).
+    try:
+        import ctypes
+        import numpy as np
+        from vision_rwkv_amd import _lib
+        L = _lib.lib()
+        L.vrwkv_wkv6_fwd_phases_bytes.restype = ctypes.c_size_t
+        L.vrwkv_wkv6_fwd_phases_bytes.argtypes = [ctypes.c_int] * 3
+        L.vrwkv_wkv6_fwd_phases.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        nb = L.vrwkv_wkv6_fwd_phases_bytes(Bw, Tw, Hw)
+        st = torch.zeros(nb // 8, dtype=torch.int64, device=dev)
+        y = torch.empty(Bw, Tw, Cw, device=dev)
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        for _ in range(3):
+            rc = L.vrwkv_wkv6_fwd_phases(P(r), P(k), P(v), P(w), P(u), P(y), Bw, Tw, Cw, Hw, P(st), nb,
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            if rc:
+                raise RuntimeError(f"vrwkv_wkv6_fwd_phases returned status {rc}")
+        torch.cuda.synchronize()
+        t = st.cpu().numpy().reshape(Bw * Hw, waves, nchunk, 8).astype(np.float64)
+        m_stage, e_stage = t[..., 5] - t[..., 4], t[..., 1] - t[..., 0]
+        step = t[:, :, 1:, 0] - t[:, :, :-1, 0]
+        busy = mfma_per_wave_step * mfma_cycles
+        out["phases"] = {
+            "unit": "shader-clock cycles per wave and chunk step (mean over all waves and steps)",
+            "matrix_stage": round(float(m_stage.mean()), 1), "elementwise_stage": round(float(e_stage.mean()), 1),
+            "whole_step": round(float(step.mean()), 1),
+            "mfma_pipe_cycles_per_wave_step": busy,
+            "mfma_busy_in_contractions": round(busy / float(m_stage.mean()), 4),
+            "mfma_busy_in_contractions_simd": round(min(1.0, 4 * busy / float(step.mean())), 4),
+            "note": "mfma_busy_in_contractions = one wave's MFMA pipe cycles / the time it spends in its matrix stage; "
+                    "..._simd = the four waves sharing a SIMD (two workgroups per CU) x their MFMA cycles / one step: "
+                    "the pipe's busy share while the kernel runs at full occupancy",
+        }
+    except Exception as e:                                  # the profiling entry is optional; the timing above stands
+        out["phases"] = {"error": repr(e)}
     # end to end the operator's arithmetic intensity (issued MFMA flop per mandatory byte) is below the machine
     # balance, so min(MFMA peak, AI x HBM peak) is the HBM leg: report the fraction of it as well
     io_bytes = Bw * Tw * Cw * (3 * r.element_size() + w.element_size() + 4) + u.numel() * 4
@@ -172,19 +237,35 @@ def backward_section(torch, ops, steps, warmup):
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(99)
     w, u = (t.to(dev) for t in baseline_wu(torch))
-    k, v, gy = (torch.randn(B, T, C, generator=g).to(dev) for _ in range(3))
     Hw = C // 64
-    r6, k6, v6 = (torch.randn(B, T, C, generator=g).to(dev).bfloat16() for _ in range(3))
-    w6 = (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(dev)
     u6 = (torch.randn(Hw, 64, generator=g) * 0.1).to(dev)
 
     def timed(fn):
         return median_us(torch, fn, steps, warmup)[0]
 
-    us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
-    kh, vh, gyh = k.bfloat16(), v.bfloat16(), gy.bfloat16()
-    us_bh = timed(lambda: ops.bi_wkv_backward(w, u, kh, vh, gyh))
-    us_6 = timed(lambda: ops.wkv6_backward(B, T, C, Hw, r6, k6, v6, w6, u6, gy))
+    # every figure on input sets in rotation (more than the last-level cache holds between two uses of a set)
+    def make_b(i):
+        return tuple(torch.randn(B, T, C, generator=g).to(dev) for _ in range(3))
+    fn, sets = rotating(make_b, 3 * B * T * C * 4, lambda k, v, gy: ops.bi_wkv_backward(w, u, k, v, gy))
+    us_b = timed(fn)
+    sets_h = [tuple(t.bfloat16() for t in s_) for s_ in sets]
+    del sets, fn
+    state = {"i": 0}
+
+    def fn_h():
+        k, v, gy = sets_h[state["i"]]
+        state["i"] = (state["i"] + 1) % len(sets_h)
+        return ops.bi_wkv_backward(w, u, k, v, gy)
+    us_bh = timed(fn_h)
+    del sets_h
+
+    def make_6(i):
+        r6, k6, v6 = (torch.randn(B, T, C, generator=g).to(dev).bfloat16() for _ in range(3))
+        return r6, k6, v6, (torch.randn(B, T, C, generator=g) * 0.5 - 0.5).to(dev), torch.randn(B, T, C, generator=g).to(dev)
+    fn6, sets6 = rotating(make_6, B * T * C * (3 * 2 + 4 + 4),
+                          lambda r6, k6, v6, w6, gy: ops.wkv6_backward(B, T, C, Hw, r6, k6, v6, w6, u6, gy))
+    us_6 = timed(fn6)
+    del sets6, fn6
     bytes_b = 5 * B * T * C * 4                                  # k, v, gy read; gk, gv written
     return {"biwkv_bwd_us_per_call": round(us_b, 2), "biwkv_bwd_GBps": round(bytes_b / (us_b * 1e-6) / 1e9, 1),
             "biwkv_bwd_pct_hbm_peak": round(100 * bytes_b / (us_b * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
@@ -203,7 +284,6 @@ def sweep_section(torch, ops, steps, warmup):
     for Bn, Tn, Cn in shapes:
         if True:
             g = torch.Generator(device="cpu").manual_seed(Tn + Cn)
-            k, v, gy = (torch.randn(Bn, Tn, Cn, generator=g).to(dev) for _ in range(3))
             c = torch.arange(Cn, dtype=torch.float32)
             w = ((-5 + 8 * c / (Cn - 1)) / Tn).to(dev)
             u = ((math.log(0.3) + 0.5 * (((c + 1) % 3) - 1)) / Tn).to(dev)
@@ -211,12 +291,29 @@ def sweep_section(torch, ops, steps, warmup):
             def timed(fn):
                 return median_us(torch, fn, steps, warmup)[0]
 
-            us_f = timed(lambda: ops.bi_wkv_forward(w, u, k, v))
-            us_b = timed(lambda: ops.bi_wkv_backward(w, u, k, v, gy))
-            kh, vh = k.bfloat16(), v.bfloat16()
-            us_h = timed(lambda: ops.bi_wkv_forward(w, u, kh, vh))
+            # input sets in rotation, more than the last-level cache holds (the small shapes need many)
+            fn, sets = rotating(lambda i: tuple(torch.randn(Bn, Tn, Cn, generator=g).to(dev) for _ in range(3)),
+                                3 * Bn * Tn * Cn * 4, lambda k, v, gy: ops.bi_wkv_forward(w, u, k, v))
+            us_f = timed(fn)
+            state = {"i": 0}
+
+            def fn_b():
+                k, v, gy = sets[state["i"]]
+                state["i"] = (state["i"] + 1) % len(sets)
+                return ops.bi_wkv_backward(w, u, k, v, gy)
+            us_b = timed(fn_b)
+            sets_h = [(k.bfloat16(), v.bfloat16()) for k, v, _ in sets]
+            n_sets = len(sets)
+            del sets, fn
+
+            def fn_h():
+                kh, vh = sets_h[state["i"] % len(sets_h)]
+                state["i"] = (state["i"] + 1) % len(sets_h)
+                return ops.bi_wkv_forward(w, u, kh, vh)
+            us_h = timed(fn_h)
+            del sets_h
             el = Bn * Tn * Cn * 4
-            rows.append({"B": Bn, "T": Tn, "C": Cn, "fwd_us": round(us_f, 1), "fwd_GBps": round(3 * el / us_f / 1e3, 1),
+            rows.append({"B": Bn, "T": Tn, "C": Cn, "input_sets": n_sets, "fwd_us": round(us_f, 1), "fwd_GBps": round(3 * el / us_f / 1e3, 1),
                          "fwd_bf16_us": round(us_h, 1), "fwd_bf16_GBps": round(3 * el / 2 / us_h / 1e3, 1),
                          "bwd_us": round(us_b, 1), "bwd_GBps": round(5 * el / us_b / 1e3, 1)})
     return rows

@@ -98,6 +98,18 @@ int vrwkv_wkv6_fwd(const void* r, const void* k, const void* v, const void* w, c
                    float* y, int B, int T, int C, int H, int rkv_dtype, int w_dtype, int w_is_ew,
                    void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* Profiling twin of vrwkv_wkv6_fwd (no counterpart in the reference; for benchmarks and tuning): the same kernel
+ * for bf16 r, k, v and fp32 raw-logit w, with every wave storing the shader clock at the boundaries of its stages.
+ * stamps: device buffer of vrwkv_wkv6_fwd_phases_bytes(B, T, H) bytes, laid out as uint64
+ * [B*H][8 waves][ceil(T/32) chunk steps][8 points]: 0 element-wise stage entered, 1 its operands written (before the
+ * barrier), 2 behind that barrier, 4 matrix stage entered, 5 y stored and the next decay sums formed (before the
+ * barrier), 6 behind that barrier; 3 and 7 unused.  Waves 0-3 are the descending pass, 4-7 the ascending one.  y is
+ * written as by vrwkv_wkv6_fwd.  Sequences whose decays fall outside the chunked kernel's range leave later steps
+ * unstamped. */
+size_t vrwkv_wkv6_fwd_phases_bytes(int B, int T, int H);
+int vrwkv_wkv6_fwd_phases(const void* r, const void* k, const void* v, const void* w, const float* u,
+                          float* y, int B, int T, int C, int H, void* stamps, size_t stamp_bytes, void* hip_stream);
+
 /* ---- wkv6 backward ---------------------------------------------------------------------
  * Replaces backward(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu)
  *   (classification/mmcls_custom/models/backbones/cuda_v6/wkv6_op.cpp:10-12, launcher

@@ -7,10 +7,10 @@
 //
 //   y_n = sum_j r_n[j] ( u[j] k_n[j] v_n  +  sum_{m<n} (prod_{m<l<n} d_l[j]) k_m[j] v_m )
 //
-// One 512-thread workgroup per (b,h): waves 0-3 run the descending pass, waves 4-7 the ascending
-// one, side by side and in lockstep (chunk step s of both passes between the same barriers); two
-// workgroups per CU put four waves on every SIMD.  Chunks of 32 tokens.  With the in-chunk cumulative
-// log-decay P_n = sum_{l<=n} log d_l (Pex_n = P_n - log d_n) and the chunk's end as the reference, P31:
+// One 512-thread workgroup per (b,h): waves 0-3 run the descending pass, waves 4-7 the ascending one, half a
+// step apart (see "schedule" in the kernel); two workgroups per CU put four waves on every SIMD.  Chunks of 32
+// tokens.  With the in-chunk cumulative log-decay P_n = sum_{l<=n} log d_l (Pex_n = P_n - log d_n) and the
+// chunk's end as the reference, P31:
 //   rt_n = r_n * exp(Pex_n - P31),   kt_m = k_m * exp(P31 - P_m)       (rt_n . kt_m = decay for m<n)
 //   A[n][m] = rt_n . kt_m  (m < n),  bonus_n = (r_n u) . k_n  (m = n, ascending pass), 0 otherwise -> MFMA 1
 //   Z       = diag(e^P31) S                                  the state as the chunk's end sees it
@@ -18,16 +18,16 @@
 //   S'      = Z + kt^T V                                                       -> MFMA 4, accumulated onto Z
 // so one scaled copy of the state serves the read-out and the update.  In the matrix stage a wave owns 16
 // value columns: S (64 x 16, four 16x16 accumulator tiles) never leaves its registers and goes straight
-// back in as the B operand of MFMA 3 -- the contraction index is taken in the order the accumulator layout
-// provides, and the rt operand is read from LDS in that same order, which is also the order MFMA 1
-// contracts in, so one set of rt registers feeds both.  Likewise A goes from the accumulators of MFMA 1
-// into the A operand of MFMA 2 (every wave forms the whole 32 x 32 A: three 16x16 blocks, the fourth is
-// masked out as a whole).
+// back in as an operand of MFMA 3 -- the contraction index is taken in the order the accumulator layout
+// provides, the [token][channel] arrays in LDS keep their channels in that same order (an operand is one
+// 16-byte read), and MFMA 1 contracts in it too, so one set of rt registers feeds both.  Likewise A goes from
+// the accumulators of MFMA 1 into an operand of MFMA 2 (every wave forms the whole 32 x 32 A: three 16x16
+// blocks, the fourth is masked out as a whole).  The y tiles are accumulated transposed, so that a lane holds
+// four neighbouring columns of a token and a tile is stored with 16-byte accesses.
 //
-// y: both passes walk the same chunk grid from opposite ends.  The pass that reaches a chunk at the
-// earlier step stores, the other one adds at its (later) step, after the barrier that ends every step (at
-// the middle chunk of an odd count the descending pass stores before that barrier and the ascending pass
-// adds after it) -- y is never zero-filled, and there is no second launch.
+// y: both passes walk the same chunk grid from opposite ends.  The pass that reaches a chunk first stores,
+// the other one fetches those values ahead of its matrix stage and accumulates on top of them -- y is never
+// zero-filled, and there is no second launch.
 //
 // Precision: every operand that is computed rather than loaded (rt, kt, A, Z) is split into a
 // bf16 head and a bf16 tail and the products head*head + head*tail + tail*head are accumulated,
@@ -352,6 +352,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             // ================================= stage M: matrix cores ===============================
             const int g4 = lane_e >> 4, c16 = lane_e & 15;                // lane = (column c16, slot group g4)
             stamp(ch, 4);
+            __builtin_amdgcn_s_setprio(2);        // the matrix stage goes first on its SIMD: its MFMA chains and LDS round trips are the long pole
             if (y_late) {
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb) accY[tb] = __builtin_bit_cast(f32x4v, BufRaw<16>::ld(rsy, y_lane, y_row(cy, tb, Cs)));
@@ -486,6 +487,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 BufRaw<16>::st(__builtin_bit_cast(typename BufRaw<16>::type, accY[tb]), rsy, y_lane, y_row(cy, tb, Cs));
             // the next chunk's decay sums (its rows were fetched at the top of this stage)
             decay_sums(ch + 1 < nchunk ? ch + 1 : ch, Cs, p);
+            __builtin_amdgcn_s_setprio(0);
             if (y_drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             stamp(ch, 5);
         }
