@@ -246,6 +246,8 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         // loop they would hold a dozen registers (128 per wave is the budget for four waves per SIMD).
         int lane_e = lane;
         asm volatile("" : "+v"(lane_e));
+        int w4s = w4, hps = hp;                                           // the same for what depends on the wave number
+        asm volatile("" : "+s"(w4s), "+s"(hps));
         const int cy = chunk_of(ch);
         // the other pass's M of chunk cy on the common clock: the descending one runs in half 2 (nchunk - cy), the
         // ascending one in half 2 cy + 1; this step's E runs in half hp, its M in half hp + 1
@@ -257,7 +259,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         const bool y_drain = (asc ? 2 * (nchunk - 1 - cy) + 1 : 2 * cy) == hp + 1;
         {
             // =============================== stage E: elementwise =================================
-            // wave w4 of the pass prepares tokens n = 8 w4 .. 8 w4 + 7 of the chunk; lane = channel j (and i for v)
+            // wave w4s of the pass prepares tokens n = 8 w4s .. 8 w4s + 7 of the chunk; lane = channel j (and i for v)
             // Column of channel j = lane_e in the [token][channel] arrays: the matrix stage contracts over the channels
             // in the order the state's accumulator tiles give (slot (g4, e) of contraction half kb <-> j = 32 kb + 4 g4 + e
             // for e < 4, 32 kb + 16 + 4 g4 + e - 4 for e >= 4), so the arrays keep the channels in that order and an
@@ -270,13 +272,13 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             // rest = log2 decay from the start of this wave's tokens to the chunk's end (P_m - P31 = p[m] - rest >= 0),
             // p31 = that of the whole chunk; the waves' totals were written at the end of the previous matrix stage
             const float t0 = L.Tot[0][lane_e], t1 = L.Tot[1][lane_e], t2 = L.Tot[2][lane_e], t3 = L.Tot[3][lane_e];
-            const float m0 = w4 == 0 ? 1.f : 0.f, m1 = w4 <= 1 ? 1.f : 0.f, m2 = w4 <= 2 ? 1.f : 0.f;     // wave-uniform
+            const float m0 = w4s == 0 ? 1.f : 0.f, m1 = w4s <= 1 ? 1.f : 0.f, m2 = w4s <= 2 ? 1.f : 0.f;     // wave-uniform
             const float rest = fmaf(m0, t0, fmaf(m1, t1, fmaf(m2, t2, t3)));
             const float p31 = (t0 + t1) + (t2 + t3);
-            if (w4 == 0 && __builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag[hp & 1] = 1;
+            if (w4s == 0 && __builtin_amdgcn_ballot_w64(!(p31 >= -SAFE_DECAY * LOG2E)) != 0ull && lane == 0) sFlag[hps & 1] = 1;
             // Z = diag(e^P31) S, in place, split into head and tail for MFMA 3 (done here, while the r, k, v rows are still
             // on their way): a lane needs e^P31 of the channels its state rows belong to, taken from the wave's own copy
-            L.C2[w4][lane_e] = fast_exp2(p31);
+            L.C2[w4s][lane_e] = fast_exp2(p31);
             {
                 const int g4 = lane_e >> 4;
 #pragma unroll
@@ -284,7 +286,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     float z8[8];
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) {
-                        const f32x4 c2 = *reinterpret_cast<const f32x4*>(&L.C2[w4][16 * (2 * kb + hf) + 4 * g4]);
+                        const f32x4 c2 = *reinterpret_cast<const f32x4*>(&L.C2[w4s][16 * (2 * kb + hf) + 4 * g4]);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { S[2 * kb + hf][e] *= c2[e]; z8[4 * hf + e] = S[2 * kb + hf][e]; }
                     }
@@ -297,7 +299,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 float zp = -rest;                                         // Pex_m - P31 = z_(m-1)
 #pragma unroll
                 for (int m = 0; m < 8; m += 2) {
-                    const int n = 8 * w4 + m;
+                    const int n = 8 * w4s + m;
                     const float z0 = p[m] - rest, z1 = p[m + 1] - rest;
                     const float f1a = fast_exp2(zp), f2a = fast_exp2(-z0);    // exp(Pex - P31), exp(P31 - P)
                     const float f1b = fast_exp2(z0), f2b = fast_exp2(-z1);
@@ -324,21 +326,21 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     pu[m] = r0 * uj * k0;
                     pu[m + 1] = r1 * uj * k1;
                 }
-                *reinterpret_cast<u32x4*>(&L.Kth[lane_e][8 * w4]) = u32x4{kthw[0], kthw[1], kthw[2], kthw[3]};
-                *reinterpret_cast<u32x4*>(&L.Ktl[lane_e][8 * w4]) = u32x4{ktlw[0], ktlw[1], ktlw[2], ktlw[3]};
-                *reinterpret_cast<u32x4*>(&L.Vt[lane_e][8 * w4]) = u32x4{vthw[0], vthw[1], vthw[2], vthw[3]};
+                *reinterpret_cast<u32x4*>(&L.Kth[lane_e][8 * w4s]) = u32x4{kthw[0], kthw[1], kthw[2], kthw[3]};
+                *reinterpret_cast<u32x4*>(&L.Ktl[lane_e][8 * w4s]) = u32x4{ktlw[0], ktlw[1], ktlw[2], ktlw[3]};
+                *reinterpret_cast<u32x4*>(&L.Vt[lane_e][8 * w4s]) = u32x4{vthw[0], vthw[1], vthw[2], vthw[3]};
                 if constexpr (VSPLIT)
-                    *reinterpret_cast<u32x4*>(&L.Vtl[lane_e][8 * w4]) = u32x4{vtlw[0], vtlw[1], vtlw[2], vtlw[3]};
+                    *reinterpret_cast<u32x4*>(&L.Vtl[lane_e][8 * w4s]) = u32x4{vtlw[0], vtlw[1], vtlw[2], vtlw[3]};
                 if (asc) {                                                // bonus_n = sum_j r_n[j] u[j] k_n[j]
                     int idx;
                     const float rs = row_sums8(pu, lane_e, idx);
-                    L.Bon[lane_e >> 4][8 * w4 + idx] = rs;                // the four 16-channel rows are added by the reader
+                    L.Bon[lane_e >> 4][8 * w4s + idx] = rs;                // the four 16-channel rows are added by the reader
                 }
             }
             // earlier y values of this chunk (none: an out-of-range offset reads 0 without a memory access)
             {
                 const int g4 = lane_e >> 4, c16 = lane_e & 15;
-                y_lane = (unsigned)(((asc ? c16 : 15 - c16) * Cs + 16 * w4 + 4 * g4) * sizeof(float));
+                y_lane = (unsigned)(((asc ? c16 : 15 - c16) * Cs + 16 * w4s + 4 * g4) * sizeof(float));
                 const unsigned vo = y_second && !y_late ? y_lane : OOB_OFFSET;
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb) accY[tb] = __builtin_bit_cast(f32x4v, BufRaw<16>::ld(rsy, vo, y_row(cy, tb, Cs)));
@@ -347,7 +349,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         }
         sync_step();
         stamp(ch, 2);
-        if (sFlag[hp & 1]) { bail = true; break; }                       // out of range: redo with the exact recurrence
+        if (sFlag[hps & 1]) { bail = true; break; }                       // out of range: redo with the exact recurrence
         {
             // ================================= stage M: matrix cores ===============================
             const int g4 = lane_e >> 4, c16 = lane_e & 15;                // lane = (column c16, slot group g4)
@@ -404,7 +406,11 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 __builtin_amdgcn_sched_barrier(0);
             }
             // ---- phase 2: operands of the products over the chunk's tokens ----
-            const int icol = 16 * w4 + c16;
+            // The next step's r, k, v rows go out first (the operand registers of the phases above are free): their latency
+            // runs behind the rest of this stage, the barrier and the first part of stage E (the last step re-reads its own
+            // rows: no branch, the compiler's wait counts stay exact).
+            fetch_rkv(ch + 1 < nchunk ? ch + 1 : ch, Cs);
+            const int icol = 16 * w4s + c16;
             const bf16x8 bv = cat8(*reinterpret_cast<const bf16x4*>(&L.Vt[icol][4 * g4]),
                                    *reinterpret_cast<const bf16x4*>(&L.Vt[icol][16 + 4 * g4]));
             const bf16x8 bs = *reinterpret_cast<const bf16x8*>(&L.Vt[icol][8 * g4]);
@@ -413,7 +419,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                 bvl = cat8(*reinterpret_cast<const bf16x4*>(&L.Vtl[icol][4 * g4]), *reinterpret_cast<const bf16x4*>(&L.Vtl[icol][16 + 4 * g4]));
                 bsl = *reinterpret_cast<const bf16x8*>(&L.Vtl[icol][8 * g4]);
             }
-            bf16x8 kth[4], ktl[4];
+            bf16x8 kth[4];
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) kth[jt] = *reinterpret_cast<const bf16x8*>(&L.Kth[16 * jt + c16][8 * g4]);
             float bon[2];
@@ -459,28 +465,26 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
             {
                 const bf16x8 Ah0 = words8(ahw[0][0], ahw[0][1], 0u, 0u), Al0 = words8(alw[0][0], alw[0][1], 0u, 0u);
                 const bf16x8 Ah1 = words8(ahw[1][0], ahw[1][1], ahw[2][0], ahw[2][1]), Al1 = words8(alw[1][0], alw[1][1], alw[2][0], alw[2][1]);
-                // the tails of kt^T are read behind the first MFMAs of this phase (their registers were A's accumulators)
-#pragma unroll
-                for (int jt = 0; jt < 4; ++jt) ktl[jt] = *reinterpret_cast<const bf16x8*>(&L.Ktl[16 * jt + c16][8 * g4]);
-                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kth[jt], bs, S[jt], 0, 0, 0);
                 accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Ah0, accY[0], 0, 0, 0);
                 accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Ah1, accY[1], 0, 0, 0);
-#pragma unroll
-                for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ktl[jt], bs, S[jt], 0, 0, 0);
-                accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al0, accY[0], 0, 0, 0);
-                accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al1, accY[1], 0, 0, 0);
                 if constexpr (VSPLIT) {
 #pragma unroll
                     for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kth[jt], bsl, S[jt], 0, 0, 0);
                     accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bvl, Ah0, accY[0], 0, 0, 0);
                     accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bvl, Ah1, accY[1], 0, 0, 0);
                 }
+                // the tails of kt^T take the heads' registers: read while the MFMAs above run
+                __builtin_amdgcn_sched_barrier(0);
+                bf16x8 ktl[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) ktl[jt] = *reinterpret_cast<const bf16x8*>(&L.Ktl[16 * jt + c16][8 * g4]);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) S[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ktl[jt], bs, S[jt], 0, 0, 0);
+                accY[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al0, accY[0], 0, 0, 0);
+                accY[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, Al1, accY[1], 0, 0, 0);
             }
-            // the next step's r, k, v rows: their latency runs behind the rest of this stage, the barrier and the first
-            // part of stage E (the last step re-reads its own rows: no branch, the compiler's wait counts stay exact)
-            fetch_rkv(ch + 1 < nchunk ? ch + 1 : ch, Cs);
             // ---- y: store (the sum with the other pass's values where it came first) ----
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
@@ -493,7 +497,7 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
         }
         sync_step();
         stamp(ch, 6);
-        if (sFlag[(hp + 1) & 1]) { bail = true; break; }
+        if (sFlag[(hps + 1) & 1]) { bail = true; break; }
     }
     if (asc && !bail) sync_step();
 
