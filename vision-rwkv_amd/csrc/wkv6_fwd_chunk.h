@@ -403,6 +403,9 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
                     accA[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KL[0], RH[tb], accA[tb], 0, 0, 0);
                 }
                 accA[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KL[1], RH[1], accA[2], 0, 0, 0);
+                // While the matrix pipe works these off, the vector ALUs form the next chunk's decay sums (its rows were
+                // fetched at the top of stage E; p and the totals of this step are no longer read).
+                if (kb == 1) decay_sums(ch + 1 < nchunk ? ch + 1 : ch, Cs, p);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // ---- phase 2: operands of the products over the chunk's tokens ----
@@ -489,8 +492,6 @@ void wkv6_fwd_chunk_kernel(const IO* __restrict__ r_, const IO* __restrict__ k_,
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
                 BufRaw<16>::st(__builtin_bit_cast(typename BufRaw<16>::type, accY[tb]), rsy, y_lane, y_row(cy, tb, Cs));
-            // the next chunk's decay sums (its rows were fetched at the top of this stage)
-            decay_sums(ch + 1 < nchunk ? ch + 1 : ch, Cs, p);
             __builtin_amdgcn_s_setprio(0);
             if (y_drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             stamp(ch, 5);
