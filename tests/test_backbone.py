@@ -325,20 +325,24 @@ def test_fused_qshift_mix_backward_against_autograd(B, Hp, Wp, C, head_dim, cls,
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("N,dtype,with_sums", [(768, torch.float32, True), (1024, torch.float32, True), (64, torch.float32, True),
-                                                (768, torch.bfloat16, True), (4096, torch.float32, False),
-                                                (3072, torch.bfloat16, False)])
-def test_row_fuse_backward_against_autograd(N, dtype, with_sums):
+@pytest.mark.parametrize("N,dtype,with_sums,rows", [
+    (768, torch.float32, True, (5, 9)), (1024, torch.float32, True, (5, 9)), (64, torch.float32, True, (5, 9)),
+    (768, torch.bfloat16, True, (5, 9)), (4096, torch.float32, False, (5, 9)), (3072, torch.bfloat16, False, (5, 9)),
+    # more rows than the grid has waves (a wave walks several rows, the last ones fewer than the first), at every
+    # vector shape the kernel picks: 8-byte x 3 (768 bf16), 16-byte x 2 (1024 bf16), 8-byte x 1 (192), 16-byte x 1 (384),
+    # fp32 16-byte x 3 and x 4
+    (768, torch.bfloat16, True, (3, 3001)), (1024, torch.bfloat16, True, (3, 2203)), (192, torch.bfloat16, True, (2, 4111)),
+    (384, torch.float16, True, (2, 4111)), (768, torch.float32, True, (3, 2203)), (1024, torch.float32, True, (3, 1409))])
+def test_row_fuse_backward_against_autograd(N, dtype, with_sums, rows):
     """Gradients of the fused row epilogues (hand-written backward kernel) against autograd through the tensor-op
-    sequence in float64 on the same inputs: every pre / LayerNorm / post combination, 45 rows (the last workgroup and
-    the last wave's run of rows are partial).  Rows longer than 1024 channels are differentiated by the kernel only
+    sequence in float64 on the same inputs: every pre / LayerNorm / post combination, on 45 rows (fewer than one row
+    per wave) and on several thousand.  Rows longer than 1024 channels are differentiated by the kernel only
     without LayerNorm and gamma.  Tolerance: 2e-4 of each gradient's scale for fp32 I/O (fast exp / rcp in the gate,
-    fp32 sums over rows), 3e-2 for bf16."""
+    fp32 sums over rows), 3e-2 for 16-bit I/O."""
     import vision_rwkv_amd as ops
     O = ops.ops
     dev = "cuda:0"
     torch.manual_seed(N)
-    rows = (5, 9)
     tol = 2e-4 if dtype == torch.float32 else 3e-2
     combos = [(O.PRE_NONE, O.POST_SIGMOID_GATE, False, False), (O.PRE_RELU_SQ, O.POST_NONE, False, False),
               (O.PRE_NONE, O.POST_RESIDUAL, False, False)]

@@ -71,7 +71,8 @@ def test_elementwise_entry_points_validate_without_device(lib):
     assert rf(one, None, None, None, None, ctypes.c_void_p(72), 4, 64, 0, 0, 1e-5, 1, None) == 1   # misaligned output
     assert rf(one, None, None, None, None, one, 4, 64, 2, 0, 1e-5, 1, None) == 1              # unknown pre
     rb = lib.vrwkv_rowfuse_bwd
-    assert lib.vrwkv_rowfuse_bwd_workspace_bytes(100, 768) == 4 * 3 * 768 * 4                # one partial row set per 32 rows
+    assert lib.vrwkv_rowfuse_bwd_workspace_bytes(100, 768) == 25 * 3 * 768 * 4               # one partial row set per workgroup
+    assert lib.vrwkv_rowfuse_bwd_workspace_bytes(1 << 20, 768) == 768 * 3 * 768 * 4         # ... of a grid of at most 768
     assert rb(one, one, None, None, None, one, one, None, None, 4, 64, 0, 1, 1e-5, 1, None, 0, None) == 1     # gate without gother
     assert rb(one, None, one, one, None, one, one, None, None, 4, 64, 0, 0, 1e-5, 1, None, 0, None) == 1      # LayerNorm without gparam
     assert rb(one, None, one, one, None, one, one, None, one, 4, 2048, 0, 0, 1e-5, 1, one, 1 << 20, None) == 3  # channel sums beyond 1024 channels

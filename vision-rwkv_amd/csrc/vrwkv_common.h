@@ -184,30 +184,32 @@ __device__ __forceinline__ void stamp(int wave, int slot, int point) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// out[c] = sum_b part[b*C + c] for up to two (part, out) pairs (the second may be null).  1024 threads = 64 columns
-// (one 256-byte piece of a row per wave load) x 16 slices of the batch, eight loads of a slice in flight at a time;
-// the slices are added in a fixed order (deterministic).  Grid: ceil(C / 64), block: BATCH_SUM_THREADS.
-constexpr int BATCH_SUM_THREADS = 1024, BATCH_SUM_COLS = 64;
+// out[c] = sum_b part[b*C + c] for up to two (part, out) pairs (the second may be null).  1024 threads = 32 columns
+// (one 128-byte piece of a row per half wave) x 32 slices of the batch, sixteen loads of a slice in flight at a time
+// (512 partial rows in one round of loads); the slices are added in a fixed order (deterministic).
+// Grid: ceil(C / BATCH_SUM_COLS), block: BATCH_SUM_THREADS.
+constexpr int BATCH_SUM_THREADS = 1024, BATCH_SUM_COLS = 32, BATCH_SUM_SLICES = BATCH_SUM_THREADS / BATCH_SUM_COLS;
 __global__ __launch_bounds__(1024) inline void batch_sum_kernel(const float* __restrict__ part0, float* __restrict__ out0,
                                                                 const float* __restrict__ part1, float* __restrict__ out1,
                                                                 int B, int C) {
-    __shared__ float red[2][16][BATCH_SUM_COLS];
-    const int cl = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    constexpr int NS = BATCH_SUM_SLICES, U = 16;
+    __shared__ float red[2][NS][BATCH_SUM_COLS];
+    const int cl = threadIdx.x % BATCH_SUM_COLS, slice = threadIdx.x / BATCH_SUM_COLS;
     const int c = blockIdx.x * BATCH_SUM_COLS + cl;
     float s0 = 0.f, s1 = 0.f;
     if (c < C) {
         int b = slice;
-        for (; b + 16 * 7 < B; b += 16 * 8) {
-            float t0[8], t1[8];
+        for (; b + NS * (U - 1) < B; b += NS * U) {
+            float t0[U], t1[U];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                t0[i] = part0[(size_t)(b + 16 * i) * C + c];
-                t1[i] = part1 ? part1[(size_t)(b + 16 * i) * C + c] : 0.f;
+            for (int i = 0; i < U; ++i) {
+                t0[i] = part0[(size_t)(b + NS * i) * C + c];
+                t1[i] = part1 ? part1[(size_t)(b + NS * i) * C + c] : 0.f;
             }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { s0 += t0[i]; s1 += t1[i]; }
+            for (int i = 0; i < U; ++i) { s0 += t0[i]; s1 += t1[i]; }
         }
-        for (; b < B; b += 16) {
+        for (; b < B; b += NS) {
             s0 += part0[(size_t)b * C + c];
             if (part1) s1 += part1[(size_t)b * C + c];
         }
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(1024) inline void batch_sum_kernel(const float* __r
     if (slice == 0 && c < C) {
         float t0 = 0.f, t1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { t0 += red[0][i][cl]; t1 += red[1][i][cl]; }
+        for (int i = 0; i < NS; ++i) { t0 += red[0][i][cl]; t1 += red[1][i][cl]; }
         out0[c] = t0;
         if (part1) out1[c] = t1;
     }
