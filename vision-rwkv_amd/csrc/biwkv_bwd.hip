@@ -63,11 +63,12 @@ struct BwdPlan {
 
 BwdPlan make_bwd_plan(int B, int T, int C) {
     BwdPlan p;
-    static const int kL[] = {4, 8, 16, 28};
+    static const int kL[] = {4, 8, 16, 25, 28};
+    const int el = option(OPT_BIWKV_L);                      // tuning override: tokens per wave
     const bool tiled = !option(OPT_BIWKV_BWD_SERIAL) && (long long)T * C < (1LL << 29);   // the option forces the sequential kernel (testing)
     if (tiled) {
-        for (int i = 3; i >= 0; --i)
-            if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX) p.L = kL[i];     // smallest L that fits: most waves per tile
+        for (int i = 4; i >= 0; --i)
+            if ((T + kL[i] - 1) / kL[i] <= BWD_SMAX && (!el || el == kL[i])) p.L = kL[i];   // smallest L that fits: most waves per tile
         if (p.L) {
             p.S = (T + p.L - 1) / p.L;
         } else {
@@ -95,7 +96,7 @@ void launch_tiled(const BwdPlan& p, const float* w, const float* u, const IO* k,
     if (grid > geo.n_tiles) grid = geo.n_tiles;
     const dim3 g(grid), blk(p.S * WAVE);
     if (p.nSC == 1) {
-        if constexpr (sizeof(IO) == 4 && L % 4 == 0) {
+        if constexpr (sizeof(IO) == 4) {
             const bool aligned = C % 4 == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
             if (aligned && !option(OPT_BIWKV_NO_STAGE)) {
                 hipLaunchKernelGGL((biwkv_bwd_tile_kernel<IO, L, 0, true>), g, blk, 0, st, w, u, k, v, gy, gk, gv, ws, agg1, agg2,
@@ -132,6 +133,7 @@ int launch(const float* w, const float* u, const void* k, const void* v, const v
         case 4:  launch_tiled<IO, 4>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
         case 8:  launch_tiled<IO, 8>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
         case 16: launch_tiled<IO, 16>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
+        case 25: launch_tiled<IO, 25>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
         case 28: launch_tiled<IO, 28>(p, w, u, kk, vv, gg, ok, ov, ws, agg1, agg2, gw_part, gu_part, B, T, C, st); break;
         default:
             hipLaunchKernelGGL((biwkv_bwd_serial_kernel<IO>), dim3((C + 63) / 64, B), dim3(64), 0, st, w, u,

@@ -98,7 +98,8 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
     __shared__ float s2[BWD_SMAX][9][WAVE];
     __shared__ float s3[BWD_SMAX][2][WAVE];
     __shared__ float s_in[MODE >= 2 ? BWD_SMAX : 1][13][WAVE];   // what other super-chunks contribute, parked per wave
-    __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? BWD_SMAX : 1][2][STAGED ? L : 1][WAVE];
+    constexpr int NI = (L + 3) / 4, LR = 4 * NI;              // staging instructions (four fp32 rows each) and LDS rows per tensor
+    __shared__ __attribute__((aligned(16))) float s_stage[STAGED ? BWD_SMAX : 1][2][STAGED ? LR : 1][WAVE];
 
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -125,12 +126,13 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
         const __amdgpu_buffer_rsrc_t rv = make_rsrc(v_ + slab, bytes);
         const int cq = ctile * WAVE + (lane & 15) * 4;
 #pragma unroll
-        for (int i = 0; i < L / 4; ++i) {
-            const int rowt = tw + 4 * i + (lane >> 4);
-            const unsigned vo = (rowt < T && cq < C) ? (unsigned)(((size_t)rowt * C + cq) * 4) : OOB_OFFSET;
+        for (int i = 0; i < NI; ++i) {
+            const int rl = 4 * i + (lane >> 4);                           // row inside this wave's chunk
+            const int rowt = tw + rl;
+            const unsigned vo = (rl < L && rowt < T && cq < C) ? (unsigned)(((size_t)rowt * C + cq) * 4) : OOB_OFFSET;
             typedef __attribute__((address_space(3))) void* lds_ptr;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)(stage + i * 256), 16, vo, 0, 0, CPOL_NT);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(stage + L * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)(stage + LR * WAVE + i * 256), 16, vo, 0, 0, CPOL_NT);
         }
     };
     // workgroups are dealt round-robin to the 8 XCDs: per round, XCD x takes a contiguous eighth of the tiles
@@ -250,7 +252,7 @@ void biwkv_bwd_tile_kernel(const float* __restrict__ w_, const float* __restrict
             for (int j = 0; j < L; ++j)                      // gy first: it must not queue behind the next tile's rows
                 Gr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rg, voff0 + (unsigned)j * row, 0);
 #pragma unroll
-            for (int j = 0; j < L; ++j) { Ks[j] = stage[j * WAVE + lane]; Vs[j] = stage[(L + j) * WAVE + lane]; }
+            for (int j = 0; j < L; ++j) { Ks[j] = stage[j * WAVE + lane]; Vs[j] = stage[(LR + j) * WAVE + lane]; }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
             if (next_tile < n_tiles) issue_stage(next_tile);
         } else {

@@ -813,7 +813,7 @@ struct Plan {
     bool multi() const { return nSC > 1; }
 };
 
-constexpr int kLs[] = {4, 8, 16, 28};
+constexpr int kLs[] = {4, 8, 16, 25, 28};
 constexpr int kNumL = sizeof(kLs) / sizeof(kLs[0]);
 
 inline int num_cus() {
@@ -830,7 +830,6 @@ inline int num_cus() {
 
 inline Plan make_plan(int B, int T, int C, int io_dtype) {
     Plan p;
-    (void)io_dtype;
     const int el = option(OPT_BIWKV_L);              // tuning overrides
     const int es = option(OPT_BIWKV_S);
     p.VEC = 1;
@@ -840,6 +839,10 @@ inline Plan make_plan(int B, int T, int C, int io_dtype) {
         if (el && L != el) continue;
         const int S = (T + L - 1) / L;
         if (S > smax_for(L, p.VEC)) continue;
+        // 25-token chunks exist for 16-bit rows of 176..200 tokens (196: eight waves, two per SIMD, where 7 x 28 leaves
+        // one SIMD a single wave; the 16-bit kernel is bound by instruction issue: 17.3 -> 16.7 us at 64 x 196 x 768)
+        if (L == 25 && !el && (S != 8 || io_dtype == VRWKV_F32)) continue;
+        if (L == 25 && !el) { best = i; break; }
         const int waste = S * L - T;
         if (waste < best_waste) { best = i; best_waste = waste; }
     }
@@ -917,7 +920,7 @@ int launch_VEC(const Plan& p, const float* w, const float* u, const void* k, con
                float* ws, int B, int T, int C, hipStream_t st) {
     switch (p.L) {
 #define VRWKV_CASE(LL) case LL: return launch_L<IO, VEC, LL>(p, w, u, k, v, y, ws, B, T, C, st); break;
-        VRWKV_CASE(4) VRWKV_CASE(8) VRWKV_CASE(16) VRWKV_CASE(28)
+        VRWKV_CASE(4) VRWKV_CASE(8) VRWKV_CASE(16) VRWKV_CASE(25) VRWKV_CASE(28)
 #undef VRWKV_CASE
     }
     set_error("biwkv_fwd: internal error, no kernel for L=%d VEC=%d", p.L, VEC);
