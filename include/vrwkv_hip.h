@@ -39,7 +39,9 @@ const char* vrwkv_last_error(void);      /* thread-local, never NULL */
 /* Tuning / testing switches, process-wide (no counterpart in the reference).  Names: "biwkv_l", "biwkv_s",
  * "biwkv_grid", "biwkv_no_stage", "biwkv_no_resident", "biwkv_bwd_serial", "wkv6_fwd_scalar", "wkv6_bwd_scalar",
  * "wkv6_bwd_unfused"; 0 = default behaviour.  The initial value of <name> is that of the environment variable
- * VRWKV_<NAME> when the library first looks at any switch; the entry points never read the environment afterwards. */
+ * VRWKV_<NAME> when the library first looks at any switch; the entry points never read the environment afterwards.
+ * vrwkv_set_option rejects (VRWKV_INVALID_ARG) a value the plans would ignore: biwkv_l takes 0, 4, 8, 16, 25, 28 (tokens
+ * per wave), biwkv_s 0 or 2..8 (waves per workgroup), biwkv_grid 0 or a positive workgroup count, the others 0 or 1. */
 int vrwkv_set_option(const char* name, int value);
 int vrwkv_get_option(const char* name, int* value);
 
@@ -64,7 +66,8 @@ int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v
  * process ends) and the call allocates nothing.  Shapes whose workspace (vrwkv_biwkv_fwd_workspace_bytes) exceeds
  * vrwkv_biwkv_fwd_static_max_workspace_bytes() are rejected with VRWKV_WORKSPACE_TOO_SMALL.  All calls on one GPU
  * share that array: calls that may overlap on a GPU (different streams or threads) race; use vrwkv_biwkv_fwd with
- * separate workspaces for those. */
+ * separate workspaces for those.  The first call on a device looks up the array's device address (hipGetSymbolAddress,
+ * which may load the code object): make it outside a stream capture; every later call only launches kernels. */
 size_t vrwkv_biwkv_fwd_static_max_workspace_bytes(void);
 int vrwkv_biwkv_fwd_static(const float* w, const float* u, const void* k, const void* v, void* y,
                            int B, int T, int C, int io_dtype, void* hip_stream);

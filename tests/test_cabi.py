@@ -35,6 +35,23 @@ def test_version_and_error_string(lib):
     assert isinstance(lib.vrwkv_last_error(), bytes)
 
 
+def test_option_values_are_validated(lib):
+    """vrwkv_set_option refuses unknown names and values the plans would silently ignore; accepted values read back."""
+    val = ctypes.c_int(-1)
+    assert lib.vrwkv_set_option(b"no_such_switch", 1) == 1
+    assert lib.vrwkv_get_option(b"no_such_switch", ctypes.byref(val)) == 1
+    for name, good, bad in ((b"biwkv_l", (4, 8, 16, 25, 28, 0), (7, 32, -1)), (b"biwkv_s", (2, 8, 0), (1, 9, -3)),
+                            (b"biwkv_grid", (64, 0), (-1,)), (b"wkv6_fwd_scalar", (1, 0), (2, -1)),
+                            (b"biwkv_bwd_serial", (1, 0), (5,))):
+        for v in good:
+            assert lib.vrwkv_set_option(name, v) == 0, (name, v)
+            assert lib.vrwkv_get_option(name, ctypes.byref(val)) == 0 and val.value == v
+        for v in bad:
+            assert lib.vrwkv_set_option(name, v) == 1, (name, v)
+            assert name in lib.vrwkv_last_error()
+            assert lib.vrwkv_get_option(name, ctypes.byref(val)) == 0 and val.value == 0     # unchanged
+
+
 def test_argument_validation_without_device(lib):
     f = lib.vrwkv_biwkv_fwd
     one = ctypes.c_void_p(16)

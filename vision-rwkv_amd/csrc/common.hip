@@ -73,6 +73,14 @@ extern "C" int vrwkv_set_option(const char* name, int value) {
         vrwkv::set_error("vrwkv_set_option: unknown option '%s'", name ? name : "(null)");
         return VRWKV_INVALID_ARG;
     }
+    bool ok = value == 0 || value == 1;
+    if (i == vrwkv::OPT_BIWKV_L) ok = value == 0 || value == 4 || value == 8 || value == 16 || value == 25 || value == 28;
+    if (i == vrwkv::OPT_BIWKV_S) ok = value == 0 || (value >= 2 && value <= 8);
+    if (i == vrwkv::OPT_BIWKV_GRID) ok = value >= 0;
+    if (!ok) {
+        vrwkv::set_error("vrwkv_set_option: %d is no value of '%s'", value, name);
+        return VRWKV_INVALID_ARG;
+    }
     (void)vrwkv::option((vrwkv::Option)i);          // the environment is read before the first change
     vrwkv::g_options[i].store(value, std::memory_order_relaxed);
     return VRWKV_OK;
