@@ -177,9 +177,6 @@ def wkv6_section(torch, ops, steps, warmup, with_cpu):
         import numpy as np
         from vision_rwkv_amd import _lib
         L = _lib.lib()
-        L.vrwkv_wkv6_fwd_phases_bytes.restype = ctypes.c_size_t
-        L.vrwkv_wkv6_fwd_phases_bytes.argtypes = [ctypes.c_int] * 3
-        L.vrwkv_wkv6_fwd_phases.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         nb = L.vrwkv_wkv6_fwd_phases_bytes(Bw, Tw, Hw)
         st = torch.zeros(nb // 8, dtype=torch.int64, device=dev)
         y = torch.empty(Bw, Tw, Cw, device=dev)

@@ -118,3 +118,38 @@ def test_error_behaviour(ops):
         ops.RUN_CUDA_RWKV6(1, 4, 64, 1, x.transpose(1, 2).contiguous().transpose(1, 2), x, x, x, u)
     with pytest.raises(RuntimeError):
         ops.wkv6_forward(1, 4, 64, 1, x.cpu(), x, x, x, u)
+
+
+def test_phase_stamping_entry_point(ops):
+    """vrwkv_wkv6_fwd_phases (the chunked kernel writing a shader-clock stamp at six points of every wave's chunk
+    steps, which bench.py turns into its per-phase figures): same y as the plain entry point bit for bit, every stamp
+    written, and the stamps of a wave in program order -- stage E entered, operands written, behind the barrier, matrix
+    stage entered, y stored, behind the barrier -- within a step and from step to step.  Also its argument checks."""
+    import ctypes
+    lib = ops.lib()
+    dev = "cuda:0"
+    B, T, H = 3, 200, 2
+    C = H * 64
+    r, k, v, w, u = gen(B, T, H, 77)
+    tt = lambda a, d: torch.from_numpy(a).to(dev).to(d)
+    rt, kt, vt, wt, ut = tt(r, torch.bfloat16), tt(k, torch.bfloat16), tt(v, torch.bfloat16), tt(w, torch.float32), tt(u, torch.float32)
+    want = ops.RUN_CUDA_RWKV6(B, T, C, H, rt, kt, vt, wt, ut)
+    nb = lib.vrwkv_wkv6_fwd_phases_bytes(B, T, H)
+    nchunk = (T + 31) // 32
+    assert nb == B * H * 8 * nchunk * 8 * 8
+    st = torch.zeros(nb // 8, dtype=torch.int64, device=dev)
+    y = torch.full((B, T, C), float("nan"), device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    args = (rt.data_ptr(), kt.data_ptr(), vt.data_ptr(), wt.data_ptr(), ut.data_ptr(), y.data_ptr(), B, T, C, H)
+    assert lib.vrwkv_wkv6_fwd_phases(*args, st.data_ptr(), nb, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y, want)
+    s = st.cpu().numpy().reshape(B * H, 8, nchunk, 8)
+    pts = s[..., [0, 1, 2, 4, 5, 6]]
+    assert (pts > 0).all()
+    assert (np.diff(pts, axis=-1) >= 0).all()                       # inside a step
+    assert (s[:, :, 1:, 0] >= s[:, :, :-1, 6]).all()                # from step to step
+    # a stamp buffer that is too small, or missing, is refused before anything is launched
+    assert lib.vrwkv_wkv6_fwd_phases(*args, st.data_ptr(), nb - 8, stream) == 5
+    assert lib.vrwkv_wkv6_fwd_phases(*args, None, nb, stream) == 1
+    assert lib.vrwkv_wkv6_fwd_phases_bytes(0, T, H) == 0

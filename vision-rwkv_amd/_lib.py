@@ -63,6 +63,10 @@ def _declare(lib):
     lib.vrwkv_wkv6_fwd_workspace_bytes.restype = sz
     lib.vrwkv_wkv6_fwd.argtypes = [vp, vp, vp, vp, fp, vp, i, i, i, i, i, i, i, vp, sz, vp]
     lib.vrwkv_wkv6_fwd.restype = i
+    lib.vrwkv_wkv6_fwd_phases_bytes.argtypes = [i, i, i]
+    lib.vrwkv_wkv6_fwd_phases_bytes.restype = sz
+    lib.vrwkv_wkv6_fwd_phases.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, vp, sz, vp]
+    lib.vrwkv_wkv6_fwd_phases.restype = i
     lib.vrwkv_wkv6_bwd_workspace_bytes.argtypes = [i, i, i, i]
     lib.vrwkv_wkv6_bwd_workspace_bytes.restype = sz
     lib.vrwkv_wkv6_bwd.argtypes = [vp, vp, vp, vp, fp, fp, fp, fp, fp, fp, fp, i, i, i, i, i, i, i, vp, sz, vp]
