@@ -494,10 +494,21 @@ def backbone_section(torch, ops, steps, warmup):
         u6 = torch.randn(H6, 64, device=dev) * 0.1
         ms_wkv6 = timed(lambda: ops.wkv6_forward(B6, 196, 768, H6, r6, k6, v6, w6, u6), 12 * steps, 12 * warmup) * 12
     # VRWKV-B (classification/configs/vrwkv/vrwkv_base_16xb64_in1k.py: 224x224, C=768, 12 blocks, post-norm, layer
-    # scale), one training forward + backward at the per-GPU batch of 64 through the HIP operators and autograd
+    # scale): the inference forward with the receptance gate inside the Bi-WKV kernel and as a pass of its own, then
+    # one training forward + backward at the per-GPU batch of 64 through the HIP operators and autograd
     netb = ops.VRWKV(img_size=224, patch_size=16, embed_dims=768, depth=12, post_norm=True, init_values=1e-5).to(dev).bfloat16()
-    netb.train()
     imgb = torch.randn(64, 3, 224, 224, device=dev, dtype=torch.bfloat16)
+    netb.eval()
+    with torch.no_grad():
+        ms_b_fwd = timed(lambda: netb(imgb), steps, warmup)
+        for m in netb.modules():
+            if hasattr(m, "fused_gate"):
+                m.fused_gate = False
+        ms_b_fwd_gate_pass = timed(lambda: netb(imgb), steps, warmup)
+        for m in netb.modules():
+            if hasattr(m, "fused_gate"):
+                m.fused_gate = True
+    netb.train()
 
     def train_step():
         netb.zero_grad(set_to_none=True)
@@ -519,6 +530,10 @@ def backbone_section(torch, ops, steps, warmup):
             "ms_per_forward_unfused_shift": round(ms_fwd_eager_shift, 3),
             "ms_per_forward_all_elementwise_in_pytorch": round(ms_fwd_unfused, 3),
             "biwkv_ms_per_forward": round(ms_wkv, 3), "biwkv_share": round(ms_wkv / ms_fwd, 4),
+            "vrwkv_b": {"workload": "VRWKV-B forward, batch 64, 224x224, T=196, C=768, 12 blocks, bf16, random weights, "
+                                    "sigmoid(r) gate inside the Bi-WKV kernel (vrwkv_biwkv_fwd_gate)",
+                        "ms_per_forward": round(ms_b_fwd, 3), "images_per_s": round(64 / ms_b_fwd * 1e3, 1),
+                        "ms_per_forward_gate_as_a_pass_of_its_own": round(ms_b_fwd_gate_pass, 3)},
             "vrwkv_b_train": {"workload": "VRWKV-B forward + backward (no optimizer step), batch 64, 224x224, T=196, C=768, "
                                           "12 blocks, bf16, random weights, Bi-WKV forward and backward on the HIP kernels",
                               "ms_per_step": round(ms_train, 3), "images_per_s": round(64 / ms_train * 1e3, 1)},

@@ -60,6 +60,19 @@ int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v
                     int B, int T, int C, int io_dtype,
                     void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* Bi-WKV forward with the receptance gate applied before y is stored: y = sigmoid(r) * wkv(w, u, k, v), i.e. the
+ * operator plus the step that follows it in VRWKV_SpatialMix.forward when key_norm is off
+ * (classification/mmcls_custom/models/backbones/vrwkv.py:183-186: rwkv = RUN_CUDA(...); rwkv = sr * rwkv).  The
+ * reference has no such entry (it runs the gate as PyTorch ops on the stored y); this one saves writing y and reading
+ * it back.  r: (B,T,C) of the dtype of k, v; every other argument as vrwkv_biwkv_fwd (same workspace).  The gate runs
+ * inside the emitting kernel for 16-byte aligned k, v, y with C a multiple of 16 bytes of elements, on the one-launch
+ * path (T <= 224) and, for 16-bit rows, the two-launch path; other calls (unaligned rows, fp32 sequences beyond 224
+ * tokens, 16-bit sequences of 225..672 tokens, which a kernel without the gate serves) run vrwkv_biwkv_fwd and then
+ * gate y in place -- same result, smaller saving.  Forward only. */
+int vrwkv_biwkv_fwd_gate(const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
+                         int B, int T, int C, int io_dtype,
+                         void* workspace, size_t workspace_bytes, void* hip_stream);
+
 /* Bi-WKV forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as vrwkv_biwkv_fwd,
  * but the long-sequence workspace is an array built into the library (4 MiB of device memory per GPU, held until the

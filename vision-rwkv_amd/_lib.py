@@ -51,6 +51,8 @@ def _declare(lib):
     lib.vrwkv_biwkv_fwd_workspace_bytes.restype = sz
     lib.vrwkv_biwkv_fwd.argtypes = [fp, fp, vp, vp, vp, i, i, i, i, vp, sz, vp]
     lib.vrwkv_biwkv_fwd.restype = i
+    lib.vrwkv_biwkv_fwd_gate.argtypes = [fp, fp, vp, vp, vp, vp, i, i, i, i, vp, sz, vp]
+    lib.vrwkv_biwkv_fwd_gate.restype = i
     lib.vrwkv_biwkv_fwd_static_max_workspace_bytes.argtypes = []
     lib.vrwkv_biwkv_fwd_static_max_workspace_bytes.restype = sz
     lib.vrwkv_biwkv_fwd_static.argtypes = [fp, fp, vp, vp, vp, i, i, i, i, vp]

@@ -156,6 +156,7 @@ class VRWKV_SpatialMix(nn.Module):
         self.receptance = nn.Linear(n_embd, n_embd, bias=False)
         self.key_norm = nn.LayerNorm(n_embd) if key_norm else None
         self.output = nn.Linear(n_embd, n_embd, bias=False)
+        self.fused_gate = True     # inference without key_norm: sigmoid(r) * y inside the Bi-WKV kernel
 
     def forward(self, x, patch_resolution):
         B, T, C = x.shape
@@ -173,6 +174,9 @@ class VRWKV_SpatialMix(nn.Module):
             w, u = eval_cached(self, "wu", (self.spatial_decay, self.spatial_first), T,
                                lambda: ((self.spatial_decay / T).float().contiguous(),
                                         (self.spatial_first / T).float().contiguous()))
+            if self.key_norm is None and self.fused_gate and r.dtype == k.dtype:
+                # the receptance gate (vrwkv.py:185-186) applied inside the operator, before y is stored
+                return _proj(self.output, bi_wkv_forward(w, u, k.contiguous(), v.contiguous(), gate=r.contiguous()))
             y = bi_wkv_forward(w, u, k.contiguous(), v.contiguous())
         y = y.to(r.dtype)
         # key_norm and the sigmoid gate (vrwkv.py:184-186) in one pass; tensor ops under autograd

@@ -6,9 +6,9 @@
 
 namespace vrwkv {
 namespace biwkv_fwd_detail {
-extern template int biwkv_fwd_launch_io<float>(const Plan&, const float*, const float*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
-extern template int biwkv_fwd_launch_io<__hip_bfloat16>(const Plan&, const float*, const float*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
-extern template int biwkv_fwd_launch_io<__half>(const Plan&, const float*, const float*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
+extern template int biwkv_fwd_launch_io<float>(const Plan&, const float*, const float*, const void*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
+extern template int biwkv_fwd_launch_io<__hip_bfloat16>(const Plan&, const float*, const float*, const void*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
+extern template int biwkv_fwd_launch_io<__half>(const Plan&, const float*, const float*, const void*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
 }
 namespace {
 using namespace biwkv_fwd_detail;
@@ -78,41 +78,124 @@ extern "C" size_t vrwkv_biwkv_fwd_workspace_bytes(int B, int T, int C, int io_dt
     return (size_t)B * p.nSC * NSLOT * C * sizeof(float);
 }
 
-extern "C" int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v, void* y,
-                               int B, int T, int C, int io_dtype,
-                               void* workspace, size_t workspace_bytes, void* hip_stream) {
+namespace vrwkv {
+namespace {
+
+// y <- sigmoid(r) * y in place: the gate as a pass of its own, for the calls whose kernels have no gated variant.
+// 16-byte pieces where both tensors allow it (two per thread in flight), single elements for the rest and the tail.
+template <typename IO>
+__global__ __launch_bounds__(256)
+void gate_in_place_kernel(const IO* r_, IO* y_, size_t n, size_t n_vec) {
+    constexpr int V = 16 / (int)sizeof(IO);
+    const size_t stride = (size_t)gridDim.x * blockDim.x, tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    auto one = [&](size_t i) {
+        float rv[V], yv[V];
+        load_vec_nt<IO, V>(r_ + i * V, rv);
+        load_vec<IO, V>(y_ + i * V, yv);
+#pragma unroll
+        for (int e = 0; e < V; ++e) yv[e] *= fast_rcp(1.f + fast_exp2(-rv[e] * LOG2E));
+        store_vec<IO, V>(y_ + i * V, yv);
+    };
+    size_t i = tid;
+    for (; i + stride < n_vec; i += 2 * stride) {
+        float r0[V], y0[V], r1[V], y1[V];
+        load_vec_nt<IO, V>(r_ + i * V, r0);
+        load_vec<IO, V>(y_ + i * V, y0);
+        load_vec_nt<IO, V>(r_ + (i + stride) * V, r1);
+        load_vec<IO, V>(y_ + (i + stride) * V, y1);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            y0[e] *= fast_rcp(1.f + fast_exp2(-r0[e] * LOG2E));
+            y1[e] *= fast_rcp(1.f + fast_exp2(-r1[e] * LOG2E));
+        }
+        store_vec<IO, V>(y_ + i * V, y0);
+        store_vec<IO, V>(y_ + (i + stride) * V, y1);
+    }
+    if (i < n_vec) one(i);
+    for (size_t j = n_vec * V + tid; j < n; j += stride) {
+        const float g = fast_rcp(1.f + fast_exp2(-to_f32(r_[j]) * LOG2E));
+        y_[j] = from_f32<IO>(to_f32(y_[j]) * g);
+    }
+}
+template <typename IO>
+int launch_gate_in_place(const void* r, void* y, size_t n, hipStream_t st) {
+    constexpr int V = 16 / (int)sizeof(IO);
+    const bool aligned = (((uintptr_t)r | (uintptr_t)y) & 15) == 0;
+    const size_t n_vec = aligned ? n / V : 0;
+    const size_t work = n_vec / 2 + (n - n_vec * V) + 1;          // threads that have something to do
+    size_t blocks = (work + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL((gate_in_place_kernel<IO>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const IO*>(r), static_cast<IO*>(y), n, n_vec);
+    return check_launch("biwkv_fwd_gate");
+}
+
+// the forward, with the gate when r is given
+int biwkv_fwd_common(const char* who, const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
+                     int B, int T, int C, int io_dtype, void* workspace, size_t workspace_bytes, void* hip_stream) {
     int rc = validate(B, T, C, io_dtype);
     if (rc != VRWKV_OK) return rc;
     if (!w || !u || !k || !v || !y) {
-        set_error("biwkv_fwd: null pointer argument");
+        set_error("%s: null pointer argument", who);
         return VRWKV_INVALID_ARG;
     }
     const size_t esz = io_dtype == VRWKV_F32 ? 4 : 2;
-    if ((((uintptr_t)k | (uintptr_t)v | (uintptr_t)y) & (esz - 1)) || (((uintptr_t)w | (uintptr_t)u) & 3)) {
-        set_error("biwkv_fwd: pointers must be aligned to their element size");
+    if ((((uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)r) & (esz - 1)) || (((uintptr_t)w | (uintptr_t)u) & 3)) {
+        set_error("%s: pointers must be aligned to their element size", who);
         return VRWKV_INVALID_ARG;
     }
     const Plan p = make_plan(B, T, C, io_dtype);
     if (p.multi()) {
         const size_t need = (size_t)B * p.nSC * NSLOT * C * sizeof(float);
         if (!workspace || workspace_bytes < need) {
-            set_error("biwkv_fwd: workspace of %zu bytes required for T=%d (got %zu)", need, T,
+            set_error("%s: workspace of %zu bytes required for T=%d (got %zu)", who, need, T,
                       workspace ? workspace_bytes : (size_t)0);
             return VRWKV_WORKSPACE_TOO_SMALL;
         }
         if ((uintptr_t)workspace & 3) {
-            set_error("biwkv_fwd: workspace must be 4-byte aligned");
+            set_error("%s: workspace must be 4-byte aligned", who);
             return VRWKV_INVALID_ARG;
         }
     }
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
     float* ws = static_cast<float*>(workspace);
+    auto go = [&](const void* rr) -> int {
+        switch (io_dtype) {
+            case VRWKV_F32:  return biwkv_fwd_launch_io<float>(p, w, u, k, v, rr, y, ws, B, T, C, st);
+            case VRWKV_BF16: return biwkv_fwd_launch_io<__hip_bfloat16>(p, w, u, k, v, rr, y, ws, B, T, C, st);
+            case VRWKV_F16:  return biwkv_fwd_launch_io<__half>(p, w, u, k, v, rr, y, ws, B, T, C, st);
+        }
+        return VRWKV_UNSUPPORTED_DTYPE;
+    };
+    rc = go(r);
+    if (rc != GATE_NOT_FUSED) return rc;
+    rc = go(nullptr);
+    if (rc != VRWKV_OK) return rc;
+    const size_t n = (size_t)B * T * C;
     switch (io_dtype) {
-        case VRWKV_F32:  return biwkv_fwd_launch_io<float>(p, w, u, k, v, y, ws, B, T, C, st);
-        case VRWKV_BF16: return biwkv_fwd_launch_io<__hip_bfloat16>(p, w, u, k, v, y, ws, B, T, C, st);
-        case VRWKV_F16:  return biwkv_fwd_launch_io<__half>(p, w, u, k, v, y, ws, B, T, C, st);
+        case VRWKV_F32:  return launch_gate_in_place<float>(r, y, n, st);
+        case VRWKV_BF16: return launch_gate_in_place<__hip_bfloat16>(r, y, n, st);
+        default:         return launch_gate_in_place<__half>(r, y, n, st);
     }
-    return VRWKV_UNSUPPORTED_DTYPE;
+}
+
+}  // namespace
+}  // namespace vrwkv
+
+extern "C" int vrwkv_biwkv_fwd(const float* w, const float* u, const void* k, const void* v, void* y,
+                               int B, int T, int C, int io_dtype,
+                               void* workspace, size_t workspace_bytes, void* hip_stream) {
+    return biwkv_fwd_common("biwkv_fwd", w, u, k, v, nullptr, y, B, T, C, io_dtype, workspace, workspace_bytes, hip_stream);
+}
+
+extern "C" int vrwkv_biwkv_fwd_gate(const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
+                                    int B, int T, int C, int io_dtype,
+                                    void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!r) {
+        set_error("biwkv_fwd_gate: null pointer argument");
+        return VRWKV_INVALID_ARG;
+    }
+    return biwkv_fwd_common("biwkv_fwd_gate", w, u, k, v, r, y, B, T, C, io_dtype, workspace, workspace_bytes, hip_stream);
 }
 
 extern "C" size_t vrwkv_biwkv_fwd_static_max_workspace_bytes(void) { return kStaticWorkspaceBytes; }

@@ -2,7 +2,7 @@
 #include "biwkv_fwd_impl.h"
 namespace vrwkv {
 namespace biwkv_fwd_detail {
-template int biwkv_fwd_launch_io<float>(const Plan&, const float*, const float*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
+template int biwkv_fwd_launch_io<float>(const Plan&, const float*, const float*, const void*, const void*, const void*, void*, float*, int, int, int, hipStream_t);
 }
 }
 #ifdef VRWKV_STAMPS

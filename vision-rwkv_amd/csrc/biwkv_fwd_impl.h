@@ -121,8 +121,11 @@ struct TileGeom {
 // STAGED (C a multiple of the 4 or 8 elements in 16 bytes, 16-byte aligned k, v, y): a tile's k, v rows are fetched as 16-byte pieces straight
 // into LDS (buffer_load ... lds, no registers, 1 KB contiguous per wave instruction instead of 256 B) while the
 // previous tile is computed, and each wave then reads its own rows back lane-per-channel.
-template <typename IO, int VEC, int L, int MODE, bool STAGED = false>
+// GATE: the emitted rows leave as sigmoid(r) * y (the receptance gate of vrwkv.py:186 applied before the store); r is
+// fetched lane-per-channel at the top of the tile, ahead of the next tile's rows, and waits packed in registers.
+template <typename IO, int VEC, int L, int MODE, bool STAGED = false, bool GATE = false>
 struct BiwkvTile {
+    static_assert(!GATE || (VEC == 1 && MODE != 1), "the gate is applied where y is emitted, one channel per lane");
     static constexpr int SMAX = smax_for(L, VEC);
     static constexpr int CH = WAVE * VEC;
     using P = Packed<IO, VEC>;
@@ -151,6 +154,7 @@ struct BiwkvTile {
     const float* __restrict__ u_;
     const IO* __restrict__ k_;
     const IO* __restrict__ v_;
+    const IO* __restrict__ r_;  // GATE: receptance (B,T,C)
     IO* __restrict__ y_;
     float* __restrict__ ws;
     int T, C;
@@ -256,6 +260,19 @@ struct BiwkvTile {
     }
     static __device__ __forceinline__ typename BufRaw<sizeof(IO) * VEC>::type load_raw(__amdgpu_buffer_rsrc_t r, unsigned vo) {
         return BufRaw<sizeof(IO) * VEC>::template ld<CPOL_NT>(r, vo, 0);
+    }
+    // GATE: this lane's r values of the tile (tokens past T read as zero and are never stored)
+    __device__ __forceinline__ void issue_gate(const Where& q, unsigned row, typename BufRaw<sizeof(IO)>::type (&Rr)[GATE ? L : 1]) const {
+        if constexpr (GATE) {
+            const __amdgpu_buffer_rsrc_t rr = make_rsrc(r_ + q.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+#pragma unroll
+            for (int j = 0; j < L; ++j) Rr[j] = BufRaw<sizeof(IO)>::template ld<CPOL_NT>(rr, q.voff0 + (unsigned)j * row, 0);
+        }
+    }
+    static __device__ __forceinline__ float gate_of(typename BufRaw<sizeof(IO)>::type raw) {
+        IO t;
+        __builtin_memcpy(&t, &raw, sizeof(t));
+        return fast_rcp(1.f + fast_exp2(-to_f32(t) * LOG2E));
     }
     __device__ __forceinline__ void issue_loads(int tile, P (&K)[L], P (&V)[L], WU& wu) const {
         issue_wu(tile, wu);
@@ -364,6 +381,7 @@ struct BiwkvTile {
         VRWKV_STAMP(wave, round, 1);                      // other super-chunks folded (MODE 2)
         // unpack; tokens past T read as zero from the buffer and get k = -inf here
         float X0[L][VEC], X1[L][VEC];                    // k / v, later E / E*v
+        typename BufRaw<sizeof(IO)>::type Rr[GATE ? L : 1];              // GATE: this lane's r, packed
         if (STAGED) {
             // This tile's rows have landed: the wait for them stands before the previous tile's first store (and
             // before the loop for the first tile).  Loads and stores share one counter and may retire in either
@@ -386,6 +404,7 @@ struct BiwkvTile {
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // rows are in registers: the region is free
             VRWKV_STAMP(wave, round, 2);                                  // rows copied from LDS
+            issue_gate(q, row, Rr);                                       // first: it must not queue behind the next tile's rows
             if (next < g.n_tiles) issue_stage(next, wun);
             VRWKV_STAMP(wave, round, 3);                                  // next tile's loads issued
         } else {
@@ -397,6 +416,7 @@ struct BiwkvTile {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) X0[j][e] = tok ? X0[j][e] : NEG_INF;
             }
+            issue_gate(q, row, Rr);
         }
 
         // ================================== fast path ==================================
@@ -580,6 +600,7 @@ struct BiwkvTile {
                 c[e] = fmaf(gd[e], c[e], X1[j][e]);
                 d[e] = fmaf(gd[e], d[e], X0[j][e]);
             }
+            if (GATE) out[0] *= gate_of(Rr[j]);
             // the next tile's rows must have landed before this tile's first store joins them in the queue
             if (STAGED && EARLY_WAIT && j == (OUT_STAGED ? 0 : L - 1)) {
                 VRWKV_STAMP(wave, round, 8);              // (16-bit: descending sweep done) waiting for the next tile's rows
@@ -743,6 +764,10 @@ struct BiwkvTile {
                 out[e] = (e1 * PN[j][e] + e2 * c[e]) / (e1 * PD[j][e] + e2 * d[e]);
                 tri_push(c[e], d[e], o[e], om[e], X0[j][e], X1[j][e]);
             }
+            if constexpr (GATE) {
+                const __amdgpu_buffer_rsrc_t rr = make_rsrc(r_ + q.slab, (unsigned)((size_t)T * C * sizeof(IO)));
+                out[0] *= gate_of(BufRaw<sizeof(IO)>::ld(rr, q.voff0 + (unsigned)j * row, 0));
+            }
             buf_store<IO, VEC>(ry, q.voff0 + (unsigned)j * row, out);
         }
         lds_barrier();
@@ -750,20 +775,20 @@ struct BiwkvTile {
 };
 
 
-template <typename IO, int VEC, int L, int MODE, bool STAGED = false>
+template <typename IO, int VEC, int L, int MODE, bool STAGED = false, bool GATE = false>
 __global__ __launch_bounds__(smax_for(L, VEC) * WAVE)
 void biwkv_fwd_kernel(const float* __restrict__ w_, const float* __restrict__ u_,
                       const IO* __restrict__ k_, const IO* __restrict__ v_, IO* __restrict__ y_,
-                      float* __restrict__ ws, int T, int C, TileGeom g)
+                      float* __restrict__ ws, int T, int C, TileGeom g, const IO* __restrict__ r_ = nullptr)
 {
-    using Tile = BiwkvTile<IO, VEC, L, MODE, STAGED>;
+    using Tile = BiwkvTile<IO, VEC, L, MODE, STAGED, GATE>;
     __shared__ float s_agg[2][Tile::SMAX][NSLOT][Tile::CH];   // fast path: slot 2 carries the wave maxima
     __shared__ __attribute__((aligned(16))) IO s_stage[STAGED ? Tile::SMAX : 1][STAGED ? Tile::STAGE_ELEMS : 1];
     __shared__ __attribute__((aligned(16))) IO s_y[Tile::OUT_STAGED ? Tile::SMAX : 1][Tile::YSTAGE_ELEMS];
     __shared__ float s_fold[MODE == 2 ? 12 : 1][WAVE];
 
     Tile t;
-    t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.y_ = y_; t.ws = ws;
+    t.w_ = w_; t.u_ = u_; t.k_ = k_; t.v_ = v_; t.r_ = r_; t.y_ = y_; t.ws = ws;
     t.T = T; t.C = C; t.g = g;
     t.lane = threadIdx.x & (WAVE - 1);
     t.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -870,21 +895,29 @@ inline Plan make_plan(int B, int T, int C, int io_dtype) {
     return p;
 }
 
+// Returned (never to the caller of the C ABI) when a gate was asked for and the kernels this call would run have no
+// gated variant: rows that cannot be staged, or the one-launch kernel for two or three super-chunks.
+constexpr int GATE_NOT_FUSED = -100;
+
+// r: null, or the receptance whose sigmoid gates y inside the emitting kernel.
 template <typename IO, int VEC, int L>
-int launch_L(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+int launch_L(const Plan& p, const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
              float* ws, int B, int T, int C, hipStream_t st) {
     const dim3 block(p.S * WAVE);
     const dim3 grid(p.grid);
     const IO* kk = static_cast<const IO*>(k);
     const IO* vv = static_cast<const IO*>(v);
+    const IO* rr = static_cast<const IO*>(r);
     IO* yy = static_cast<IO*>(y);
     // fp32 rows are staged through LDS in 16-byte pieces when the layout allows it
     if constexpr (VEC == 1) {
         const bool aligned = C % (16 / (int)sizeof(IO)) == 0 && (((uintptr_t)k | (uintptr_t)v | (uintptr_t)y) & 15) == 0;
         if (aligned && !option(OPT_BIWKV_NO_STAGE)) {
             if (!p.multi()) {
-                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+                if (rr) hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
+                else hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
             } else if (sizeof(IO) == 2 && L == 28 && p.nSC <= 3 && !option(OPT_BIWKV_NO_RESIDENT)) {
+                if (rr) return GATE_NOT_FUSED;
                 // two or three super-chunks of 16-bit rows fit a workgroup's registers: one launch, k and v read once
                 if constexpr (sizeof(IO) == 2 && L == 28) {
                     const int n_seq = B * p.geom.n_ctile;
@@ -900,26 +933,36 @@ int launch_L(const Plan& p, const float* w, const float* u, const void* k, const
 #undef VRWKV_RESIDENT
                 }
             } else {
-                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
-                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+                // fp32 rows: the emitting kernel of long sequences has no registers left for r (measured at 2 x 4150 x 768:
+                // 61 us with the gate inside against 50 us with the gate as a pass of its own); 16-bit rows: 32 against 37 us
+                if (rr && sizeof(IO) == 4) return GATE_NOT_FUSED;
+                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
+                if constexpr (sizeof(IO) == 2) {
+                    if (rr) {
+                        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2, true, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
+                        return check_launch("biwkv_fwd");
+                    }
+                }
+                hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2, true>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
             }
             return check_launch("biwkv_fwd");
         }
     }
+    if (rr) return GATE_NOT_FUSED;
     if (!p.multi()) {
-        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 0>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
     } else {
-        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
-        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom);
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 1>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
+        hipLaunchKernelGGL((biwkv_fwd_kernel<IO, VEC, L, 2>), grid, block, 0, st, w, u, kk, vv, yy, ws, T, C, p.geom, rr);
     }
     return check_launch("biwkv_fwd");
 }
 
 template <typename IO, int VEC>
-int launch_VEC(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+int launch_VEC(const Plan& p, const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
                float* ws, int B, int T, int C, hipStream_t st) {
     switch (p.L) {
-#define VRWKV_CASE(LL) case LL: return launch_L<IO, VEC, LL>(p, w, u, k, v, y, ws, B, T, C, st); break;
+#define VRWKV_CASE(LL) case LL: return launch_L<IO, VEC, LL>(p, w, u, k, v, r, y, ws, B, T, C, st); break;
         VRWKV_CASE(4) VRWKV_CASE(8) VRWKV_CASE(16) VRWKV_CASE(25) VRWKV_CASE(28)
 #undef VRWKV_CASE
     }
@@ -928,9 +971,9 @@ int launch_VEC(const Plan& p, const float* w, const float* u, const void* k, con
 }
 
 template <typename IO>
-int biwkv_fwd_launch_io(const Plan& p, const float* w, const float* u, const void* k, const void* v, void* y,
+int biwkv_fwd_launch_io(const Plan& p, const float* w, const float* u, const void* k, const void* v, const void* r, void* y,
                         float* ws, int B, int T, int C, hipStream_t st) {
-    return launch_VEC<IO, 1>(p, w, u, k, v, y, ws, B, T, C, st);
+    return launch_VEC<IO, 1>(p, w, u, k, v, r, y, ws, B, T, C, st);
 }
 
 }  // namespace biwkv_fwd_detail

@@ -38,14 +38,17 @@ def _stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def bi_wkv_forward(w, u, k, v, out=None):
+def bi_wkv_forward(w, u, k, v, out=None, gate=None):
     """Extension-level entry (bi_wkv.cpp:23-33): w,u (C,) fp32; k,v (B,T,C) of one dtype
     (fp32, bf16 or fp16); returns y (B,T,C) of that dtype.  State and arithmetic are fp32.
-    out: a caller-allocated y (the legacy interface, wkv_op.cpp:6-8)."""
-    for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v")):
+    out: a caller-allocated y (the legacy interface, wkv_op.cpp:6-8).
+    gate: None, or the receptance r (B,T,C) of the same dtype: the result is sigmoid(r) * y, the step that follows the
+    operator in VRWKV_SpatialMix.forward (vrwkv.py:185-186 without key_norm), applied before y is stored
+    (vrwkv_biwkv_fwd_gate; forward only: it has no autograd)."""
+    for t, n in ((w, "w"), (u, "u"), (k, "k"), (v, "v")) + (((gate, "gate"),) if gate is not None else ()):
         _check_input(t, n)
-    if k.dim() != 3 or v.shape != k.shape:
-        raise RuntimeError("k and v must both be (B,T,C)")
+    if k.dim() != 3 or v.shape != k.shape or (gate is not None and (gate.shape != k.shape or gate.dtype != k.dtype)):
+        raise RuntimeError("k and v (and the gate) must all be (B,T,C) of one dtype")
     B, T, C = k.shape
     if w.numel() != C or u.numel() != C:
         raise RuntimeError("w and u must have C elements")
@@ -61,9 +64,12 @@ def bi_wkv_forward(w, u, k, v, out=None):
     ws_bytes = L.vrwkv_biwkv_fwd_workspace_bytes(B, T, C, dt)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=k.device) if ws_bytes else None
     with torch.cuda.device(k.device):
-        _lib.check(L.vrwkv_biwkv_fwd(w.data_ptr(), u.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
-                                     B, T, C, dt, ws.data_ptr() if ws is not None else None, ws_bytes,
-                                     _stream_ptr(k.device)))
+        tail = (B, T, C, dt, ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(k.device))
+        if gate is None:
+            _lib.check(L.vrwkv_biwkv_fwd(w.data_ptr(), u.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(), *tail))
+        else:
+            _lib.check(L.vrwkv_biwkv_fwd_gate(w.data_ptr(), u.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(),
+                                              y.data_ptr(), *tail))
     return y
 
 
