@@ -7,8 +7,14 @@ Each function restates, row by row, a short PyTorch-op sequence of the reference
   maa_mix           .../vrwkv6.py:178-194  (xx = shift(x) - x;  x + xx * (time_maa_i + m_i), i = w, k, v, r, g)
   groupnorm_gate    .../vrwkv6.py:199, 205-211  (ln_x = GroupNorm(n_head, C) on the (B*T, C) view, times silu(gate))
 
+  spatial_mix, channel_mix, block   a whole VRWKV block composed of the above, the q_shift loops and an operator passed
+                    in by the caller: .../vrwkv.py:156-188 (VRWKV_SpatialMix), :244-262 (VRWKV_ChannelMix),
+                    :296-313 (Block: post- or pre-norm, with or without layer scale)
+
 Pinned by tests/test_oracle_blocks.py: hand-computed rows, LayerNorm / GroupNorm against torch.nn.functional in
-float64 on the CPU, and the gate / residual algebra on values chosen so that a wrong order of the steps shows.
+float64 on the CPU, the gate / residual algebra on values chosen so that a wrong order of the steps shows, and the
+composed block against the same sequence written with torch float64 tensor ops and slice-copy shifts (every variant of
+norm placement, layer scale and key_norm; identity-projection special cases by hand).
 """
 import numpy as np
 
@@ -71,3 +77,66 @@ def groupnorm_gate(y, gate, weight, bias, n_groups, eps=1e-5):
             out[i, h * G:(h + 1) * G] = (seg - mean) / np.sqrt(var + eps) * w[h * G:(h + 1) * G] + b[h * G:(h + 1) * G]
         out[i] *= gt[i] / (1.0 + np.exp(-gt[i]))                               # silu
     return out.reshape(y.shape)
+
+
+def _linear(x, weight):
+    """nn.Linear without bias: x (..., in) times weight (out, in) transposed."""
+    return np.asarray(x, np.float64) @ np.asarray(weight, np.float64).T
+
+
+def _mix(x, xx, m):
+    m = np.asarray(m, np.float64).reshape(1, 1, -1)
+    return x * m + xx * (1.0 - m)                                         # vrwkv.py:161-163, 249-250
+
+
+def spatial_mix(x, P, patch_resolution, wkv, shift_pixel=1, gamma=0.25, eps=1e-5):
+    """VRWKV_SpatialMix.forward (vrwkv.py:156-188).  x (B,T,C); P: parameters by the reference's names
+    (spatial_mix_k/v/r, key.weight, value.weight, receptance.weight, output.weight, spatial_decay, spatial_first and,
+    with key_norm, key_norm.weight / key_norm.bias); wkv(w, u, k, v) -> y is the Bi-WKV operator to use."""
+    from .qshift import q_shift_loops
+    x = np.asarray(x, np.float64)
+    B, T, C = x.shape
+    xx = q_shift_loops(x, shift_pixel, gamma, patch_resolution) if shift_pixel > 0 else x
+    xk, xv, xr = (_mix(x, xx, P[n]) if shift_pixel > 0 else x for n in ("spatial_mix_k", "spatial_mix_v", "spatial_mix_r"))
+    k, v, r = _linear(xk, P["key.weight"]), _linear(xv, P["value.weight"]), _linear(xr, P["receptance.weight"])
+    y = np.asarray(wkv(np.asarray(P["spatial_decay"], np.float64) / T, np.asarray(P["spatial_first"], np.float64) / T, k, v),
+                   np.float64)                                            # vrwkv.py:183
+    has_norm = "key_norm.weight" in P
+    y = row_epilogue(y, r, P["key_norm.weight"] if has_norm else None, P["key_norm.bias"] if has_norm else None,
+                     None, PRE_NONE, POST_SIGMOID_GATE, eps).reshape(B, T, C)   # vrwkv.py:184-186
+    return _linear(y, P["output.weight"])
+
+
+def channel_mix(x, P, patch_resolution, shift_pixel=1, gamma=0.25, eps=1e-5):
+    """VRWKV_ChannelMix.forward (vrwkv.py:244-262); P: spatial_mix_k/r, key.weight (hidden, C), value.weight (C, hidden),
+    receptance.weight and, with key_norm, key_norm.weight / key_norm.bias (hidden)."""
+    from .qshift import q_shift_loops
+    x = np.asarray(x, np.float64)
+    B, T, C = x.shape
+    xx = q_shift_loops(x, shift_pixel, gamma, patch_resolution) if shift_pixel > 0 else x
+    xk, xr = (_mix(x, xx, P[n]) if shift_pixel > 0 else x for n in ("spatial_mix_k", "spatial_mix_r"))
+    k = _linear(xk, P["key.weight"])
+    has_norm = "key_norm.weight" in P
+    k = row_epilogue(k, None, P["key_norm.weight"] if has_norm else None, P["key_norm.bias"] if has_norm else None,
+                     None, PRE_RELU_SQ, POST_NONE, eps).reshape(B, T, -1)       # square(relu(k)), key_norm
+    kv = _linear(k, P["value.weight"])
+    return row_epilogue(kv, _linear(xr, P["receptance.weight"]), post=POST_SIGMOID_GATE).reshape(B, T, C)
+
+
+def block(x, P, patch_resolution, wkv, layer_id, post_norm, shift_pixel=1, gamma=0.25, eps=1e-5):
+    """Block.forward (vrwkv.py:296-313) without drop path.  P holds the block's parameters by the reference's names
+    (ln0.* for layer 0, ln1.*, ln2.*, att.*, ffn.*, and gamma1 / gamma2 when the block has layer scale)."""
+    x = np.asarray(x, np.float64)
+    B, T, C = x.shape
+    sub = lambda prefix: {n[len(prefix):]: a for n, a in P.items() if n.startswith(prefix)}
+    ln = lambda a, n: row_epilogue(a, None, P[n + ".weight"], P[n + ".bias"], eps=eps).reshape(B, T, C)
+    if layer_id == 0:
+        x = ln(x, "ln0")
+    for branch, norm, g in (("att", "ln1", "gamma1"), ("ffn", "ln2", "gamma2")):
+        def run(inp):
+            if branch == "att":
+                return spatial_mix(inp, sub("att."), patch_resolution, wkv, shift_pixel, gamma, eps)
+            return channel_mix(inp, sub("ffn."), patch_resolution, shift_pixel, gamma, eps)
+        out = ln(run(x), norm) if post_norm else run(ln(x, norm))
+        x = row_epilogue(out, x, None, None, P.get(g), PRE_NONE, POST_RESIDUAL).reshape(B, T, C)
+    return x

@@ -263,3 +263,50 @@ def test_vrwkv_l_full_depth_batch_32_fused_against_tensor_ops(ops, monkeypatch):
         assert errs[f"out{i}"] <= 3e-2, errs
     # branch outputs after 23 blocks of slightly different inputs, each a chain of bf16 GEMMs
     assert errs["att"] <= 6e-2 and errs["ffn"] <= 6e-2, errs
+
+
+@pytest.mark.parametrize("variant", ["vrwkv_l", "vrwkv_b"])
+def test_blocks_against_the_block_oracle(ops, variant):
+    """One block of a configuration against oracle/blocks.block -- the reference's Block / VRWKV_SpatialMix /
+    VRWKV_ChannelMix (vrwkv.py:156-188, 244-262, 296-313) restated in NumPy float64 with the q_shift index loops and the
+    C oracle's Bi-WKV recurrence inside, independent of this build's backbone modules.
+      vrwkv_l: C=1024, hidden 4096, T=576 (24x24), key_norm, post-norm, layer scale (configuration 4); blocks 0 (with
+               ln0) and 1.
+      vrwkv_b: C=768, T=196 (14x14), no key_norm, post-norm, layer scale; in eval mode this block takes the Bi-WKV
+               entry point with the receptance gate inside the kernel.
+    fp32 on the GPU (fused kernels, fp32 GEMMs) against float64: 5e-5 of the output's rms-floored scale (measured
+    0.6e-5 ... 1.1e-5); bf16 against the oracle on the bf16-rounded parameters and input: 6e-2 (measured 3.0e-2 ...
+    3.8e-2: the worst of 1.2 M values at the end of a chain of bf16 GEMMs, as for the branch outputs of the two-block
+    test above)."""
+    from oracle import blocks, clib
+    import vision_rwkv_amd.backbone as bb
+    torch.manual_seed(7)
+    if variant == "vrwkv_l":
+        C, res, kw = 1024, (24, 24), dict(hidden_rate=4, init_values=0.5, post_norm=True, key_norm=True)
+    else:
+        C, res, kw = 768, (14, 14), dict(hidden_rate=4, init_values=0.5, post_norm=True, key_norm=False)
+    T = res[0] * res[1]
+    wkv = lambda w, u, k, v: clib.biwkv_fwd(np.asarray(w, np.float32), np.asarray(u, np.float32),
+                                            np.asarray(k, np.float32), np.asarray(v, np.float32))
+    for layer_id in (0, 1):
+        blk = bb.Block(C, 24, layer_id, **kw).eval()
+        with torch.no_grad():
+            for n, prm in blk.named_parameters():      # parameters away from their 1 / 0 / 0.5 defaults
+                if n.endswith("bias"):
+                    prm.normal_(0, 0.1)
+                elif n.startswith(("ln", "att.key_norm", "ffn.key_norm", "gamma")):
+                    prm.uniform_(0.5, 1.5)
+        x = torch.randn(2, T, C)
+        for dtype, tol in ((torch.float32, 5e-5), (torch.bfloat16, 6e-2)):
+            print(f"block oracle {variant} layer {layer_id} {dtype}", flush=True)
+            b16 = copy.deepcopy(blk).to(DEV).to(dtype)
+            xin = x.to(DEV).to(dtype)
+            with torch.no_grad():
+                got = b16(xin, res).float().cpu().numpy()
+            P = {n: v.detach().float().cpu().numpy().reshape(-1) if v.dim() == 3 else v.detach().float().cpu().numpy()
+                 for n, v in b16.state_dict().items()}
+            want = blocks.block(xin.float().cpu().numpy(), P, res, wkv, layer_id, kw["post_norm"])
+            err = rel_err(got, want)
+            print(f"  rel_err {err:.3e}")
+            assert np.isfinite(got).all()
+            assert err <= tol, (variant, layer_id, dtype, err)

@@ -72,3 +72,127 @@ def test_groupnorm_gate_against_torch_and_by_hand():
     got = blocks.groupnorm_gate(np.array([[1.0, 3.0, 10.0, 20.0]]), np.array([[0.0, 40.0, 40.0, 40.0]]),
                                 np.array([1.0, 2.0, 3.0, 4.0]), np.array([0.0, 1.0, 0.0, -1.0]), 2, eps=0.0)
     assert np.allclose(got, [[0.0, 40.0 * 3.0, 40.0 * -3.0, 40.0 * 3.0]], rtol=1e-12, atol=0)
+
+
+def _torch_block(x, P, res, layer_id, post_norm, key_norm, shift_pixel=1, gamma=0.25):
+    """The block written a second time, with torch float64 tensor ops and the slice-copy shift of vrwkv.py:68-79, and
+    the softmax form of the operator (y_t = sum_i W[t,i] v_i / sum_i W[t,i], W[t,i] = exp(k_i - w(|t-i|-1)), exp(u+k_t))."""
+    tt = {n: torch.from_numpy(np.asarray(a, np.float64)) for n, a in P.items()}
+    B, T, C = x.shape
+
+    def shift(a):
+        Hp, Wp = res
+        Cc = a.shape[2]
+        i = a.transpose(1, 2).reshape(B, Cc, Hp, Wp)
+        o = torch.zeros_like(i)
+        g1, g2, g3, g4 = (int(Cc * gamma * q) for q in (1, 2, 3, 4))
+        s = shift_pixel
+        o[:, 0:g1, :, s:Wp] = i[:, 0:g1, :, 0:Wp - s]
+        o[:, g1:g2, :, 0:Wp - s] = i[:, g1:g2, :, s:Wp]
+        o[:, g2:g3, s:Hp, :] = i[:, g2:g3, 0:Hp - s, :]
+        o[:, g3:g4, 0:Hp - s, :] = i[:, g3:g4, s:Hp, :]
+        o[:, g4:] = i[:, g4:]
+        return o.flatten(2).transpose(1, 2)
+
+    def wkv(w, u, k, v):
+        idx = torch.arange(T)
+        dist = (idx[:, None] - idx[None, :]).abs().double() - 1.0
+        logw = k[:, None, :, :] - w[None, None, None, :] * dist[None, :, :, None]           # (B, t, i, C)
+        eye = torch.eye(T, dtype=torch.bool)[None, :, :, None]
+        logw = torch.where(eye, (u[None, None, :] + k)[:, None, :, :].expand(B, T, T, C), logw)
+        return (torch.softmax(logw, dim=2) * v[:, None, :, :]).sum(2)
+
+    def att(a):
+        xx = shift(a)
+        mk, mv, mr = (tt["att.spatial_mix_" + n].reshape(1, 1, -1) for n in "kvr")
+        k = F.linear(a * mk + xx * (1 - mk), tt["att.key.weight"])
+        v = F.linear(a * mv + xx * (1 - mv), tt["att.value.weight"])
+        r = F.linear(a * mr + xx * (1 - mr), tt["att.receptance.weight"])
+        y = wkv(tt["att.spatial_decay"] / T, tt["att.spatial_first"] / T, k, v)
+        if key_norm:
+            y = F.layer_norm(y, (C,), tt["att.key_norm.weight"], tt["att.key_norm.bias"], 1e-5)
+        return F.linear(torch.sigmoid(r) * y, tt["att.output.weight"])
+
+    def ffn(a):
+        xx = shift(a)
+        mk, mr = (tt["ffn.spatial_mix_" + n].reshape(1, 1, -1) for n in "kr")
+        k = torch.square(torch.relu(F.linear(a * mk + xx * (1 - mk), tt["ffn.key.weight"])))
+        if key_norm:
+            k = F.layer_norm(k, (k.shape[-1],), tt["ffn.key_norm.weight"], tt["ffn.key_norm.bias"], 1e-5)
+        return torch.sigmoid(F.linear(a * mr + xx * (1 - mr), tt["ffn.receptance.weight"])) * F.linear(k, tt["ffn.value.weight"])
+
+    ln = lambda a, n: F.layer_norm(a, (C,), tt[n + ".weight"], tt[n + ".bias"], 1e-5)
+    h = torch.from_numpy(np.asarray(x, np.float64))
+    if layer_id == 0:
+        h = ln(h, "ln0")
+    for f, n, g in ((att, "ln1", "gamma1"), (ffn, "ln2", "gamma2")):
+        out = ln(f(h), n) if post_norm else f(ln(h, n))
+        h = h + (tt[g] * out if g in tt else out)
+    return h.numpy()
+
+
+def _block_params(rng, C, hidden, key_norm, layer_scale, layer_id):
+    P = {}
+    for n in ("ln1", "ln2") + (("ln0",) if layer_id == 0 else ()):
+        P[n + ".weight"], P[n + ".bias"] = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.2, C)
+    for n in "kvr":
+        P["att.spatial_mix_" + n] = rng.uniform(0, 1, C)
+    for n in "kr":
+        P["ffn.spatial_mix_" + n] = rng.uniform(0, 1, C)
+    for n in ("key", "value", "receptance", "output"):
+        P[f"att.{n}.weight"] = rng.normal(0, C ** -0.5, (C, C))
+    P["att.spatial_decay"], P["att.spatial_first"] = rng.uniform(-5, 3, C), rng.uniform(-1, 1, C)
+    P["ffn.key.weight"] = rng.normal(0, C ** -0.5, (hidden, C))
+    P["ffn.value.weight"] = rng.normal(0, hidden ** -0.5, (C, hidden))
+    P["ffn.receptance.weight"] = rng.normal(0, C ** -0.5, (C, C))
+    if key_norm:
+        P["att.key_norm.weight"], P["att.key_norm.bias"] = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.2, C)
+        P["ffn.key_norm.weight"], P["ffn.key_norm.bias"] = rng.uniform(0.5, 1.5, hidden), rng.normal(0, 0.2, hidden)
+    if layer_scale:
+        P["gamma1"], P["gamma2"] = rng.uniform(0.2, 1.0, C), rng.uniform(0.2, 1.0, C)
+    return P
+
+
+def test_block_composition_against_torch_ops_in_every_variant():
+    """oracle.blocks.block (loops, row epilogues, q_shift loops, the operator oracle's recurrence) against the same
+    block written with torch float64 ops, slice-copy shifts and the operator's softmax form: a swapped mix, a norm on
+    the wrong side of the branch, a gate before the norm or a missing 1/T on the decays would each show."""
+    from oracle import biwkv
+    rng = np.random.default_rng(11)
+    B, res, C, hidden = 2, (3, 4), 16, 40
+    T = res[0] * res[1]
+    wkv = lambda w, u, k, v: biwkv.biwkv_scan(np.asarray(w), np.asarray(u), np.asarray(k), np.asarray(v))
+    for layer_id in (0, 1):
+        for post_norm in (False, True):
+            for key_norm in (False, True):
+                for layer_scale in (False, True):
+                    P = _block_params(rng, C, hidden, key_norm, layer_scale, layer_id)
+                    x = rng.standard_normal((B, T, C))
+                    got = blocks.block(x, P, res, wkv, layer_id, post_norm)
+                    want = _torch_block(x, P, res, layer_id, post_norm, key_norm)
+                    assert np.allclose(got, want, rtol=0, atol=1e-10), (layer_id, post_norm, key_norm, layer_scale)
+
+
+def test_block_special_cases_by_hand():
+    """Identity projections, mixes of one (no shifted share), constant decay zero: the spatial mix is sigmoid(x) times
+    the plain mean-like weighting of x itself, and with u = 0, w = 0 every token weighs e^{k_i}: y_t = sum e^{x_i} x_i /
+    sum e^{x_i} for all t."""
+    from oracle import biwkv
+    B, res, C = 1, (2, 2), 4
+    T = 4
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B, T, C))
+    eye = np.eye(C)
+    P = {"spatial_mix_k": np.ones(C), "spatial_mix_v": np.ones(C), "spatial_mix_r": np.ones(C), "key.weight": eye,
+         "value.weight": eye, "receptance.weight": eye, "output.weight": eye, "spatial_decay": np.zeros(C),
+         "spatial_first": np.zeros(C)}
+    wkv = lambda w, u, k, v: biwkv.biwkv_scan(np.asarray(w), np.asarray(u), np.asarray(k), np.asarray(v))
+    got = blocks.spatial_mix(x, P, res, wkv)
+    # w = 0: decay^(|t-i|-1) = 1 for i != t, and e^{u + k_t} = e^{k_t} for i = t
+    y = (np.exp(x) * x).sum(1, keepdims=True) / np.exp(x).sum(1, keepdims=True)
+    want = y / (1.0 + np.exp(-x))
+    assert np.allclose(got, want, rtol=0, atol=1e-12)
+    # channel mix with identity key / value (hidden = C), no key_norm: sigmoid(x) * relu(x)^2
+    Pf = {"spatial_mix_k": np.ones(C), "spatial_mix_r": np.ones(C), "key.weight": eye, "value.weight": eye,
+          "receptance.weight": eye}
+    assert np.allclose(blocks.channel_mix(x, Pf, res), np.maximum(x, 0) ** 2 / (1.0 + np.exp(-x)), rtol=0, atol=1e-12)
