@@ -10,6 +10,9 @@ Each function restates, row by row, a short PyTorch-op sequence of the reference
   spatial_mix, channel_mix, block   a whole VRWKV block composed of the above, the q_shift loops and an operator passed
                     in by the caller: .../vrwkv.py:156-188 (VRWKV_SpatialMix), :244-262 (VRWKV_ChannelMix),
                     :296-313 (Block: post- or pre-norm, with or without layer scale)
+  spatial_mix_v6, block_v6          the VRWKV6 block: .../vrwkv6.py:175-228 (VRWKV_SpatialMix_V6: data-dependent mixes
+                    and decay through the low-rank tanh bottlenecks, wkv6, key_norm, ln_x, silu gate, output),
+                    :271-286 (its channel mix: the VRWKV one with the per-head shift), :314-332 (Block)
 
 Pinned by tests/test_oracle_blocks.py: hand-computed rows, LayerNorm / GroupNorm against torch.nn.functional in
 float64 on the CPU, the gate / residual algebra on values chosen so that a wrong order of the steps shows, and the
@@ -137,6 +140,58 @@ def block(x, P, patch_resolution, wkv, layer_id, post_norm, shift_pixel=1, gamma
             if branch == "att":
                 return spatial_mix(inp, sub("att."), patch_resolution, wkv, shift_pixel, gamma, eps)
             return channel_mix(inp, sub("ffn."), patch_resolution, shift_pixel, gamma, eps)
+        out = ln(run(x), norm) if post_norm else run(ln(x, norm))
+        x = row_epilogue(out, x, None, None, P.get(g), PRE_NONE, POST_RESIDUAL).reshape(B, T, C)
+    return x
+
+
+def spatial_mix_v6(x, P, patch_resolution, wkv6, n_head, shift_pixel=1, with_cls_token=False, eps=1e-5):
+    """VRWKV_SpatialMix_V6.forward (vrwkv6.py:175-228).  P: time_maa_x/w/k/v/r/g (C,), time_maa_w1 (C, 160),
+    time_maa_w2 (5, 32, C), time_decay (C,), time_decay_w1 (C, 64), time_decay_w2 (64, C), time_faaaa (H, 64),
+    key/value/receptance/gate/output .weight, ln_x.weight / ln_x.bias and, with key_norm, key_norm.*;
+    wkv6(r, k, v, w, u, H) -> y is the operator to use (w: the raw decay logit, as RUN_CUDA_RWKV6 takes it)."""
+    from .qshift import q_shift_multihead_loops
+    x = np.asarray(x, np.float64)
+    B, T, C = x.shape
+    f = lambda n: np.asarray(P[n], np.float64)
+    sx = q_shift_multihead_loops(x, shift_pixel, C // n_head, patch_resolution, with_cls_token)
+    xx = sx - x                                                                   # :178-179
+    xxx = x + xx * f("time_maa_x").reshape(-1)
+    lo = np.tanh(xxx @ f("time_maa_w1")).reshape(B * T, 5, -1).transpose(1, 0, 2)  # (5, B*T, 32), :181-182
+    m = np.einsum("fnd,fdc->fnc", lo, f("time_maa_w2")).reshape(5, B, T, C)       # :184-186
+    xw, xk, xv, xr, xg = maa_mix(x, sx, m, [f("time_maa_" + n) for n in "wkvrg"])  # :188-192
+    r, k, v = _linear(xr, P["receptance.weight"]), _linear(xk, P["key.weight"]), _linear(xv, P["value.weight"])
+    gate = _linear(xg, P["gate.weight"])                                          # silu applied by groupnorm_gate, :197
+    w = f("time_decay").reshape(-1) + np.tanh(xw @ f("time_decay_w1")) @ f("time_decay_w2")   # :199-201
+    y = np.asarray(wkv6(r, k, v, w, f("time_faaaa"), n_head), np.float64)         # :217
+    if "key_norm.weight" in P:
+        y = row_epilogue(y, None, P["key_norm.weight"], P["key_norm.bias"], eps=eps).reshape(B, T, C)
+    y = groupnorm_gate(y, gate, P["ln_x.weight"], P["ln_x.bias"], n_head, eps).reshape(B, T, C)   # :205-211
+    return _linear(y, P["output.weight"])
+
+
+def block_v6(x, P, patch_resolution, wkv6, n_head, layer_id, post_norm, shift_pixel=1, with_cls_token=False, eps=1e-5):
+    """Block.forward of vrwkv6.py:314-332 without drop path; parameters by the reference's names as in `block`."""
+    from .qshift import q_shift_multihead_loops
+    x = np.asarray(x, np.float64)
+    B, T, C = x.shape
+    sub = lambda prefix: {n[len(prefix):]: a for n, a in P.items() if n.startswith(prefix)}
+    ln = lambda a, n: row_epilogue(a, None, P[n + ".weight"], P[n + ".bias"], eps=eps).reshape(B, T, C)
+
+    def ffn(inp):                                                                 # vrwkv6.py:271-286
+        Pf = sub("ffn.")
+        xx = q_shift_multihead_loops(inp, shift_pixel, C // n_head, patch_resolution, with_cls_token)
+        k = _linear(_mix(inp, xx, Pf["spatial_mix_k"]), Pf["key.weight"])
+        has_norm = "key_norm.weight" in Pf
+        k = row_epilogue(k, None, Pf["key_norm.weight"] if has_norm else None, Pf["key_norm.bias"] if has_norm else None,
+                         None, PRE_RELU_SQ, POST_NONE, eps).reshape(B, T, -1)
+        return row_epilogue(_linear(k, Pf["value.weight"]), _linear(_mix(inp, xx, Pf["spatial_mix_r"]), Pf["receptance.weight"]),
+                            post=POST_SIGMOID_GATE).reshape(B, T, C)
+
+    att = lambda inp: spatial_mix_v6(inp, sub("att."), patch_resolution, wkv6, n_head, shift_pixel, with_cls_token, eps)
+    if layer_id == 0:
+        x = ln(x, "ln0")
+    for run, norm, g in ((att, "ln1", "gamma1"), (ffn, "ln2", "gamma2")):
         out = ln(run(x), norm) if post_norm else run(ln(x, norm))
         x = row_epilogue(out, x, None, None, P.get(g), PRE_NONE, POST_RESIDUAL).reshape(B, T, C)
     return x

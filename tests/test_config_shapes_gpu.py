@@ -310,3 +310,45 @@ def test_blocks_against_the_block_oracle(ops, variant):
             print(f"  rel_err {err:.3e}")
             assert np.isfinite(got).all()
             assert err <= tol, (variant, layer_id, dtype, err)
+
+
+def test_vrwkv6_blocks_against_the_block_oracle(ops):
+    """Two VRWKV6-B blocks (C=768, 12 heads, T=196 = 14x14, hidden 3072; the classification configuration of
+    vrwkv6.py) against oracle/blocks.block_v6: the reference's VRWKV_SpatialMix_V6 / VRWKV_ChannelMix / Block restated
+    in NumPy float64 with the per-head shift loops and the C oracle's wkv6 recurrence inside (vrwkv6.py:175-228,
+    271-286, 314-332).  The low-rank mix and decay matrices are drawn at 1e-2 instead of the initial 1e-4 so that the
+    data-dependent parts carry weight.  fp32 on the GPU against float64: 1e-4 (measured 0.4e-5 and 3.4e-5; the wkv6
+    kernel's split-bf16 products are the largest term); bf16: 6e-2 of the output's scale (measured 1.2e-2, 3.6e-2), as
+    for the VRWKV blocks."""
+    from oracle import blocks, clib
+    import vision_rwkv_amd.backbone6 as b6
+    torch.manual_seed(9)
+    C, H, res = 768, 12, (14, 14)
+    T = res[0] * res[1]
+    wk = lambda r, k, v, w, u, Hh: clib.wkv6_fwd(*(np.asarray(a, np.float32) for a in (r, k, v, w, u)), Hh)
+    for layer_id, post_norm, scale in ((0, False, None), (1, True, 0.5)):
+        blk = b6.Block6(C, H, 12, layer_id, init_values=scale, post_norm=post_norm).eval()
+        with torch.no_grad():
+            for n, prm in blk.named_parameters():
+                if n.endswith("bias"):
+                    prm.normal_(0, 0.1)
+                elif n.startswith(("ln", "att.ln_x", "gamma")):
+                    prm.uniform_(0.5, 1.5)
+                elif n.endswith(("_w1", "_w2")):
+                    prm.normal_(0, 1e-2)
+        x = torch.randn(2, T, C)
+        for dtype, tol in ((torch.float32, 1e-4), (torch.bfloat16, 6e-2)):
+            print(f"block oracle vrwkv6_b layer {layer_id} {dtype}", flush=True)
+            bd = copy.deepcopy(blk).to(DEV).to(dtype)
+            xin = x.to(DEV).to(dtype)
+            with torch.no_grad():
+                got = bd(xin, res).float().cpu().numpy()
+            P = {}
+            for n, v in bd.state_dict().items():
+                a = v.detach().float().cpu().numpy()
+                P[n] = a.reshape(-1) if (a.ndim == 3 and a.shape[0] == 1) else a
+            want = blocks.block_v6(xin.float().cpu().numpy(), P, res, wk, H, layer_id, post_norm)
+            err = rel_err(got, want)
+            print(f"  rel_err {err:.3e}")
+            assert np.isfinite(got).all()
+            assert err <= tol, (layer_id, dtype, err)

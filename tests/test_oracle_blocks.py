@@ -196,3 +196,110 @@ def test_block_special_cases_by_hand():
     Pf = {"spatial_mix_k": np.ones(C), "spatial_mix_r": np.ones(C), "key.weight": eye, "value.weight": eye,
           "receptance.weight": eye}
     assert np.allclose(blocks.channel_mix(x, Pf, res), np.maximum(x, 0) ** 2 / (1.0 + np.exp(-x)), rtol=0, atol=1e-12)
+
+
+def _torch_block_v6(x, P, res, H, layer_id, post_norm, key_norm, with_cls):
+    """The VRWKV6 block a second time: torch float64 ops as vrwkv6.py writes them, the slice-copy per-head shift of
+    vrwkv6.py:75-100, and the operator as a plain token loop over a (H, 64, 64) state in both directions."""
+    tt = {n: torch.from_numpy(np.asarray(a, np.float64)) for n, a in P.items()}
+    B, T, C = x.shape
+    hd = C // H
+
+    def shift(a, s=1):
+        cls = a[:, -1:, :] if with_cls else None
+        body = a[:, :-1, :] if with_cls else a
+        Hp, Wp = res
+        i = body.transpose(1, 2).reshape(B, -1, hd, Hp, Wp)
+        o = torch.zeros_like(i)
+        q = hd // 4
+        o[:, :, 0:q, :, s:Wp] = i[:, :, 0:q, :, 0:Wp - s]
+        o[:, :, q:2 * q, :, 0:Wp - s] = i[:, :, q:2 * q, :, s:Wp]
+        o[:, :, 2 * q:3 * q, s:Hp, :] = i[:, :, 2 * q:3 * q, 0:Hp - s, :]
+        o[:, :, 3 * q:4 * q, 0:Hp - s, :] = i[:, :, 3 * q:4 * q, s:Hp, :]
+        o = o.reshape(B, C, -1).transpose(1, 2)
+        return torch.cat((o, cls), dim=1) if with_cls else o
+
+    def wkv6(r, k, v, w, u):
+        d = torch.exp(-torch.exp(w)).reshape(B, T, H, hd)
+        r, k, v = (a.reshape(B, T, H, hd) for a in (r, k, v))
+        y = torch.zeros(B, T, H, hd, dtype=torch.float64)
+        for order, bonus in ((range(T), True), (range(T - 1, -1, -1), False)):
+            S = torch.zeros(B, H, hd, hd, dtype=torch.float64)                      # S[j, i]
+            for t in order:
+                kv = k[:, t, :, :, None] * v[:, t, :, None, :]
+                y[:, t] += torch.einsum("bhj,bhji->bhi", r[:, t], (u[None, :, :, None] * kv if bonus else 0) + S)
+                S = d[:, t, :, :, None] * S + kv
+        return y.reshape(B, T, C)
+
+    def att(a):
+        sx = shift(a)
+        xx = sx - a
+        xxx = a + xx * tt["att.time_maa_x"]
+        lo = torch.tanh(xxx @ tt["att.time_maa_w1"]).view(B * T, 5, -1).transpose(0, 1)
+        mw, mk, mv, mr, mg = torch.bmm(lo, tt["att.time_maa_w2"]).view(5, B, T, -1).unbind(0)
+        xw, xk, xv, xr, xg = (a + xx * (tt["att.time_maa_" + n] + m) for n, m in zip("wkvrg", (mw, mk, mv, mr, mg)))
+        r, k, v = F.linear(xr, tt["att.receptance.weight"]), F.linear(xk, tt["att.key.weight"]), F.linear(xv, tt["att.value.weight"])
+        g = F.silu(F.linear(xg, tt["att.gate.weight"]))
+        w = tt["att.time_decay"] + torch.tanh(xw @ tt["att.time_decay_w1"]) @ tt["att.time_decay_w2"]
+        y = wkv6(r, k, v, w, tt["att.time_faaaa"])
+        if key_norm:
+            y = F.layer_norm(y, (C,), tt["att.key_norm.weight"], tt["att.key_norm.bias"], 1e-5)
+        y = F.group_norm(y.reshape(B * T, C), H, tt["att.ln_x.weight"], tt["att.ln_x.bias"], 1e-5).view(B, T, C)
+        return F.linear(y * g, tt["att.output.weight"])
+
+    def ffn(a):
+        xx = shift(a)
+        mk, mr = tt["ffn.spatial_mix_k"], tt["ffn.spatial_mix_r"]
+        k = torch.square(torch.relu(F.linear(a * mk + xx * (1 - mk), tt["ffn.key.weight"])))
+        if key_norm:
+            k = F.layer_norm(k, (k.shape[-1],), tt["ffn.key_norm.weight"], tt["ffn.key_norm.bias"], 1e-5)
+        return torch.sigmoid(F.linear(a * mr + xx * (1 - mr), tt["ffn.receptance.weight"])) * F.linear(k, tt["ffn.value.weight"])
+
+    ln = lambda a, n: F.layer_norm(a, (C,), tt[n + ".weight"], tt[n + ".bias"], 1e-5)
+    h = torch.from_numpy(np.asarray(x, np.float64))
+    if layer_id == 0:
+        h = ln(h, "ln0")
+    for f, n, g in ((att, "ln1", "gamma1"), (ffn, "ln2", "gamma2")):
+        out = ln(f(h), n) if post_norm else f(ln(h, n))
+        h = h + (tt[g] * out if g in tt else out)
+    return h.numpy()
+
+
+def test_vrwkv6_block_composition_against_torch_ops():
+    """oracle.blocks.block_v6 (maa_mix, groupnorm_gate, row epilogues, the per-head shift loops and the operator
+    oracle's recurrence) against the block written with torch float64 ops and a plain state loop for the operator:
+    norm placement, layer scale, key_norm, a class token, and the order of the five mixes."""
+    from oracle import wkv6 as o6
+    rng = np.random.default_rng(23)
+    B, res, H = 2, (2, 3), 2
+    C, hidden = H * 64, 3 * H * 64
+    wk = lambda r, k, v, w, u, Hh: o6.wkv6_scan(r, k, v, w, u, Hh)
+    for layer_id, post_norm, key_norm, layer_scale, with_cls in ((0, True, False, True, False), (1, False, True, False, True),
+                                                                 (1, True, True, True, True), (0, False, False, False, False)):
+        T = res[0] * res[1] + (1 if with_cls else 0)
+        P = {}
+        for n in ("ln1", "ln2") + (("ln0",) if layer_id == 0 else ()):
+            P[n + ".weight"], P[n + ".bias"] = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.2, C)
+        for n in "xwkvrg":
+            P["att.time_maa_" + n] = rng.uniform(0, 1, C)
+        P["att.time_maa_w1"], P["att.time_maa_w2"] = rng.normal(0, 0.1, (C, 160)), rng.normal(0, 0.1, (5, 32, C))
+        P["att.time_decay"] = rng.uniform(-3, 0.5, C)
+        P["att.time_decay_w1"], P["att.time_decay_w2"] = rng.normal(0, 0.1, (C, 64)), rng.normal(0, 0.1, (64, C))
+        P["att.time_faaaa"] = rng.normal(0, 0.3, (H, 64))
+        for n in ("key", "value", "receptance", "gate", "output"):
+            P[f"att.{n}.weight"] = rng.normal(0, C ** -0.5, (C, C))
+        P["att.ln_x.weight"], P["att.ln_x.bias"] = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.2, C)
+        P["ffn.spatial_mix_k"], P["ffn.spatial_mix_r"] = rng.uniform(0, 1, C), rng.uniform(0, 1, C)
+        P["ffn.key.weight"] = rng.normal(0, C ** -0.5, (hidden, C))
+        P["ffn.value.weight"] = rng.normal(0, hidden ** -0.5, (C, hidden))
+        P["ffn.receptance.weight"] = rng.normal(0, C ** -0.5, (C, C))
+        if key_norm:
+            P["att.key_norm.weight"], P["att.key_norm.bias"] = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.2, C)
+            P["ffn.key_norm.weight"], P["ffn.key_norm.bias"] = rng.uniform(0.5, 1.5, hidden), rng.normal(0, 0.2, hidden)
+        if layer_scale:
+            P["gamma1"], P["gamma2"] = rng.uniform(0.2, 1.0, C), rng.uniform(0.2, 1.0, C)
+        x = rng.standard_normal((B, T, C))
+        got = blocks.block_v6(x, P, res, wk, H, layer_id, post_norm, with_cls_token=with_cls)
+        want = _torch_block_v6(x, P, res, H, layer_id, post_norm, key_norm, with_cls)
+        assert np.allclose(got, want, rtol=0, atol=1e-9), (layer_id, post_norm, key_norm, layer_scale, with_cls,
+                                                            np.abs(got - want).max())
