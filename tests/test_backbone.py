@@ -332,7 +332,10 @@ def test_fused_qshift_mix_backward_against_autograd(B, Hp, Wp, C, head_dim, cls,
     # vector shape the kernel picks: 8-byte x 3 (768 bf16), 16-byte x 2 (1024 bf16), 8-byte x 1 (192), 16-byte x 1 (384),
     # fp32 16-byte x 3 and x 4
     (768, torch.bfloat16, True, (3, 3001)), (1024, torch.bfloat16, True, (3, 2203)), (192, torch.bfloat16, True, (2, 4111)),
-    (384, torch.float16, True, (2, 4111)), (768, torch.float32, True, (3, 2203)), (1024, torch.float32, True, (3, 1409))])
+    (384, torch.float16, True, (2, 4111)), (768, torch.float32, True, (3, 2203)), (1024, torch.float32, True, (3, 1409)),
+    # row lengths that leave the last group of lanes partly idle, one row, one vector per row
+    (72, torch.bfloat16, True, (1, 1)), (200, torch.float16, True, (1, 513)), (1000, torch.bfloat16, True, (1, 33)),
+    (520, torch.float32, True, (1, 7)), (4, torch.float32, True, (1, 4100))])
 def test_row_fuse_backward_against_autograd(N, dtype, with_sums, rows):
     """Gradients of the fused row epilogues (hand-written backward kernel) against autograd through the tensor-op
     sequence in float64 on the same inputs: every pre / LayerNorm / post combination, on 45 rows (fewer than one row
