@@ -165,3 +165,37 @@ def test_chunked_scans_and_sequential_sweeps_full_size(ops, force):
     want = wkv6.wkv6_grads_closed(f(r), f(k), f(v), f(w), u[:1].cpu().numpy(), 1, f(gy))
     for i, name in enumerate(("gr", "gk", "gv", "gw")):
         assert rel_err(got[i][:1, :, :64].cpu().numpy(), want[i]) <= TOL, name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,H,w_lo,w_hi,gw_tol", [
+    (3, 577, 12, -6.0, -1.0, 6e-4),      # the range VRWKV6 initialises its decay logits in (vrwkv6.py:157-161)
+    (2, 400, 4, -8.0, 0.5, 2e-3),
+    (2, 577, 4, -3.0, 1.2, 5e-3), (1, 1000, 3, -3.0, 1.2, 5e-3)])
+def test_uniform_decay_ranges_on_long_sequences(ops, B, T, H, w_lo, w_hi, gw_tol, dtype):
+    """Forward and every gradient on sequences of 400..1000 tokens with decay logits drawn uniformly from a range,
+    against the C oracle on the inputs as the kernel sees them.  y, gr, gk, gv, gu: 1e-4 of the tensor's scale, for
+    every range.  gw = ld * (running difference of two sums over the rest of the sequence): the error of the running
+    difference grows like sqrt(T) and is multiplied by |ld| = exp(w), so its bound depends on the range --
+    6e-4 for logits in [-6, -1], 5e-3 for logits up to 1.2 (a decay of 0.036 per token)."""
+    from oracle import clib
+    rng = np.random.default_rng(T + H)
+    C = H * 64
+    r, k, v, gy = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
+    k *= 0.5
+    w = rng.uniform(w_lo, w_hi, (B, T, C)).astype(np.float32)
+    u = (0.5 * rng.standard_normal((H, 64))).astype(np.float32)
+    dev = "cuda:0"
+    t = lambda a, d=torch.float32: torch.from_numpy(a).to(dev).to(d)
+    rt, kt, vt, wt, ut, gt = t(r, dtype), t(k, dtype), t(v, dtype), t(w), t(u), t(gy)
+    y = ops.wkv6_forward(B, T, C, H, rt, kt, vt, wt, ut)
+    grads = ops.wkv6_backward(B, T, C, H, rt, kt, vt, wt, ut, gt)
+    torch.cuda.synchronize()
+    f = lambda x: x.float().cpu().numpy()
+    err = {"y": rel_err(f(y), clib.wkv6_fwd(f(rt), f(kt), f(vt), w, u, H))}
+    want = clib.wkv6_bwd(f(rt), f(kt), f(vt), w, u, gy, H)
+    for name, got, ref in zip(("gr", "gk", "gv", "gw", "gu"), grads, want):
+        err[name] = rel_err(f(got), ref)
+    print("  " + ", ".join(f"{n} {e:.1e}" for n, e in err.items()), flush=True)
+    for name, e in err.items():
+        assert e <= (gw_tol if name == "gw" else 1e-4), (name, e)
