@@ -465,8 +465,29 @@ def test_split_weight_gradient_of_the_block_projections():
     z.backward(gz)
     refw = x.detach().float().reshape(-1, 192).t() @ gz.float().reshape(-1, 40)
     assert ((w.grad.float() - refw).abs().max() / refw.abs().max()).item() <= 4e-3
+    # the stacked low-rank matrices of VRWKV6 (vrwkv6.py:184-185): x (5, B*T, 32) as the transposed view the block forms
+    lo = (torch.randn(8 * 1024, 5, 32, device=dev) * 0.3).bfloat16().transpose(0, 1).requires_grad_(True)
+    w2 = (torch.randn(5, 32, 192, device=dev) * 0.05).bfloat16().requires_grad_(True)
+    m1 = bb._bmm(lo, w2)
+    assert "SplitKBmm" in type(m1.grad_fn).__name__
+    gm = torch.randn_like(m1)
+    m1.backward(gm)
+    glo1, gw21 = lo.grad.clone(), w2.grad.clone()
+    lo.grad = None
+    w2.grad = None
+    m2 = torch.bmm(lo, w2)
+    m2.backward(gm)
+    assert torch.equal(m1, m2) and torch.equal(glo1, lo.grad)
+    refw2 = torch.bmm(lo.detach().float().transpose(1, 2), gm.float())
+    err_split = ((gw21.float() - refw2).abs().max() / refw2.abs().max()).item()
+    err_plain = ((w2.grad.float() - refw2).abs().max() / refw2.abs().max()).item()
+    assert err_split <= max(2 * err_plain, 4e-3), (err_split, err_plain)
+    # the partial products are added by one sum over 16-bit values: it accumulates in fp32 and rounds once
+    part = torch.randn(8, 320, 192, device=dev).bfloat16()
+    assert torch.equal(part.sum(0), part.sum(0, dtype=torch.float32).to(torch.bfloat16))
     # plain paths
     small = torch.randn(2, 16, 192, device=dev).bfloat16().requires_grad_(True)
     assert "SplitK" not in type(bb._proj(lin, small).grad_fn).__name__
+    assert "SplitK" not in type(bb._bmm(lo[:, :64], w2).grad_fn).__name__
     with torch.no_grad():
         assert bb._proj(lin, x).grad_fn is None

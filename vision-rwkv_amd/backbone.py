@@ -79,7 +79,7 @@ class _SplitKLinear(torch.autograd.Function):
             g2, x2 = g.reshape(-1, g.shape[-1]), x.reshape(-1, x.shape[-1])
             M = g2.shape[0]
             part = torch.bmm(g2.view(S, M // S, -1).transpose(1, 2), x2.view(S, M // S, -1))
-            gw = part.sum(0, dtype=torch.float32).to(weight.dtype)    # partial products added in fp32
+            gw = part.sum(0)              # one kernel: the sum of 16-bit values accumulates in fp32 and is rounded once
         return gx, gw, None
 
 
@@ -102,8 +102,45 @@ class _SplitKMatmul(torch.autograd.Function):
             g2, x2 = g.reshape(-1, g.shape[-1]), x.reshape(-1, x.shape[-1])
             M = g2.shape[0]
             part = torch.bmm(x2.view(S, M // S, -1).transpose(1, 2), g2.view(S, M // S, -1))
-            gw = part.sum(0, dtype=torch.float32).to(weight.dtype)    # partial products added in fp32
+            gw = part.sum(0)              # accumulated in fp32, rounded once
         return gx, gw, None
+
+
+class _SplitKBmm(torch.autograd.Function):
+    """torch.bmm(x, W) for a stack of parameter matrices W (n, in, out) and x (n, M, in) with M = all B*T tokens: each
+    weight gradient x_i^T g_i is split over the tokens like _SplitKMatmul's (the library runs the deep, narrow
+    contraction on a handful of workgroups otherwise)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, splits):
+        ctx.save_for_backward(x, weight)
+        ctx.splits = splits
+        return torch.bmm(x, weight)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        S = ctx.splits
+        gx = torch.bmm(g, weight.transpose(1, 2)) if ctx.needs_input_grad[0] else None
+        gw = None
+        if ctx.needs_input_grad[1]:
+            n, M, _ = x.shape
+            x4 = x.reshape(n, S, M // S, x.shape[-1])
+            g4 = g.reshape(n, S, M // S, g.shape[-1])
+            part = torch.matmul(x4.transpose(2, 3), g4)               # (n, S, in, out)
+            gw = part.sum(1)              # accumulated in fp32, rounded once
+        return gx, gw, None
+
+
+def _bmm(x, weight):
+    """torch.bmm(x, weight) for stacked low-rank parameter matrices; split weight gradient under autograd with many
+    tokens."""
+    if (x.is_cuda and torch.is_grad_enabled() and weight.requires_grad and x.dtype == weight.dtype
+            and x.dtype in (torch.bfloat16, torch.float16) and weight.dim() == 3 and x.dim() == 3):
+        M = x.shape[1]
+        if M >= 4096 and M % 8 == 0:
+            return _SplitKBmm.apply(x, weight, 8)
+    return torch.bmm(x, weight)
 
 
 def _matmul(x, weight):

@@ -10,7 +10,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .backbone import VRWKV, eval_cached, _proj, _matmul
+from .backbone import VRWKV, eval_cached, _proj, _matmul, _bmm
 from .ops import (HEAD_SIZE, RUN_CUDA_RWKV6, q_shift, q_shift_mix, q_shift_mix_autograd, stack_mixes, row_fuse, maa_mix, groupnorm_gate, PRE_NONE, PRE_RELU_SQ, POST_NONE,
                   POST_SIGMOID_GATE, POST_RESIDUAL)
 
@@ -86,7 +86,7 @@ class VRWKV_SpatialMix_V6(nn.Module):
                                  self.shift_pixel, patch_resolution, self.with_cls_token, self.fused_shift,
                                  (self.time_maa_x,))
         lo = torch.tanh(_matmul(xxx, self.time_maa_w1)).view(B * T, 5, -1).transpose(0, 1)
-        m = torch.bmm(lo, self.time_maa_w2).view(5, B, T, C)
+        m = _bmm(lo, self.time_maa_w2).view(5, B, T, C)
         # xw..xg = x + (sx - x) * (time_maa_* + m_*)  (vrwkv6.py:190-194): one pass at inference
         maas = (self.time_maa_w, self.time_maa_k, self.time_maa_v, self.time_maa_r, self.time_maa_g)
         table = None
