@@ -293,12 +293,18 @@ def test_vrwkv6_mix_kernels_against_oracle(B, T, C, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,Hp,Wp,C,head_dim,cls,dtype", [(2, 3, 5, 16, 0, False, torch.float32), (2, 14, 14, 192, 0, False, torch.float32),
                                                            (1, 7, 9, 22, 0, False, torch.float32), (2, 6, 4, 128, 64, True, torch.float32),
-                                                           (2, 14, 14, 768, 0, False, torch.bfloat16), (3, 5, 3, 8, 0, False, torch.float32)])
+                                                           (2, 14, 14, 768, 0, False, torch.bfloat16), (3, 5, 3, 8, 0, False, torch.float32),
+                                                           # many images: fewer, longer token chunks per workgroup (three
+                                                           # chunks of 34 tokens; the whole image of 100 / 101 tokens)
+                                                           (150, 10, 10, 256, 0, False, torch.bfloat16),
+                                                           (300, 10, 10, 768, 0, False, torch.float32),
+                                                           (240, 10, 10, 512, 64, True, torch.float16)])
 def test_fused_qshift_mix_backward_against_autograd(B, Hp, Wp, C, head_dim, cls, dtype):
     """Gradients of the fused q_shift + mix (hand-written backward kernel) against autograd through the tensor-op
     formulation evaluated in float64 on the same inputs: grad of x and of every mix vector, three / two / one mix,
-    per-head quarters with a trailing class token, a channel count that forces the scalar path.
-    Tolerance: 1e-5 of the gradient's scale for fp32 I/O, 2e-2 for bf16 (one rounding of gx, bf16 inputs)."""
+    per-head quarters with a trailing class token, a channel count that forces the scalar path, batches large enough
+    for the kernel to take long token chunks.
+    Tolerance: 1e-5 of the gradient's scale for fp32 I/O, 2e-2 for 16-bit I/O (one rounding of gx, 16-bit inputs)."""
     import vision_rwkv_amd as ops
     from vision_rwkv_amd.backbone6 import q_shift_multihead
     dev = "cuda:0"

@@ -96,8 +96,10 @@ void qshift_mix_kernel(const IO* __restrict__ x_, const float* __restrict__ mix_
     }
 }
 
+constexpr int QS_TOK = 2;              // tokens a thread has in flight (three or four measure the same)
 constexpr int QS_CX = 32, QS_TY = 8;   // backward workgroup: 32 channel vectors x 8 token lanes
-constexpr int QS_TCH = 32;             // tokens per workgroup (one partial gmix row per chunk): 4 per thread
+constexpr int QS_TCH = 32;             // fewest tokens per workgroup (the workspace holds one partial gmix row per 32 tokens)
+constexpr int QS_TARGET_WG = 896;      // workgroups per launch the token chunks are sized for: one round on 256 compute units
 
 // direction of a channel vector and the token offsets of its source (forward) / destination (backward)
 __device__ __forceinline__ int qs_dir(int c, int g, int head_dim) {
@@ -145,29 +147,25 @@ void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) { mu[m][e] = cok ? mix_[(size_t)m * C + c + e] : 0.f; acc[m][e] = 0.f; }
     const size_t slab = (size_t)b * T * C + c;
-    // the chunk's tokens, evened out over the chunks (196 tokens: seven chunks of 28); a thread takes every eighth,
-    // two at a time: the sixteen loads of a pair are issued before the first value is used and wait packed
+    // the chunk's tokens, evened out over the chunks (196 tokens in two chunks: 98 each); a thread takes every eighth,
+    // two at a time: the loads of a pair are issued before the first value is used and wait packed
     const int tch = (T + n_tchunk - 1) / n_tchunk;
     const int t_begin = tc * tch, t_end = min(T, t_begin + tch);
     using Packed = typename RawVec<sizeof(IO) * VEC>::type;
     if (cok) {
+        for (int t0 = t_begin + ty; t0 < t_end; t0 += QS_TOK * QS_TY) {
+            Packed pxs[QS_TOK], pgt[QS_TOK][NMIX], pgd[QS_TOK][NMIX];
+            float keep_d[QS_TOK];
+            int tt[QS_TOK];
 #pragma unroll
-        for (int i0 = 0; i0 < QS_TCH / QS_TY; i0 += 2) {
-            Packed pxs[2], pxx[2], pgt[2][NMIX], pgd[2][NMIX];
-            float keep_s[2], keep_d[2];
-            int tt[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int t = t_begin + ty + QS_TY * (i0 + j);
+            for (int j = 0; j < QS_TOK; ++j) {
+                const int t = t0 + QS_TY * j;
                 tt[j] = t < t_end ? t : -1;
                 const int tl = t < t_end ? t : t_begin;          // a token past the chunk: load a valid one, use nothing
-                const int ts = qs_src(tl, dir, Hp, Wp, shift, n_grid_tokens);
                 const int td = qs_dst(tl, dir, Hp, Wp, shift, n_grid_tokens);
-                // neighbours outside the grid are read from the token itself and masked: no divergent branches
-                keep_s[j] = ts >= 0 ? 1.f : 0.f;
+                // a neighbour outside the grid is read from the token itself and masked: no divergent branches
                 keep_d[j] = td >= 0 ? 1.f : 0.f;
                 pxs[j] = load_packed<IO, VEC>(x_ + slab + (size_t)tl * C);
-                pxx[j] = load_packed<IO, VEC>(x_ + slab + (size_t)(ts >= 0 ? ts : tl) * C);
 #pragma unroll
                 for (int m = 0; m < NMIX; ++m) {
                     pgt[j][m] = load_packed<IO, VEC>(gs[m] + slab + (size_t)tl * C);
@@ -175,11 +173,10 @@ void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ 
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < QS_TOK; ++j) {
                 if (tt[j] < 0) continue;
-                float xs[VEC], xx[VEC], gx[VEC];
+                float xs[VEC], gx[VEC];
                 widen_packed<IO, VEC>(pxs[j], xs);
-                widen_packed<IO, VEC>(pxx[j], xx);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) gx[e] = 0.f;
 #pragma unroll
@@ -189,8 +186,14 @@ void qshift_mix_bwd_kernel(const IO* __restrict__ x_, const float* __restrict__ 
                     widen_packed<IO, VEC>(pgd[j][m], gd);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        gx[e] = fmaf(gt[e], mu[m][e], fmaf(keep_d[j] * gd[e], 1.f - mu[m][e], gx[e]));
-                        acc[m][e] = fmaf(gt[e], xs[e] - keep_s[j] * xx[e], acc[m][e]);
+                        // out_m[t] = x[t] mu + x[src(t)] (1 - mu):  x[t] reaches out_m[t] with weight mu and out_m[dst(t)]
+                        // with weight 1 - mu, so with D = g_m[dst(t)] (0 outside the grid)
+                        //   gx[t] += D + (g_m[t] - D) mu,   gmix_m += x[t] (g_m[t] - D)
+                        // (the second one is the sum over t of g_m[t] (x[t] - x[src(t)]) re-indexed by the source token)
+                        const float D = keep_d[j] * gd[e];
+                        const float diff = gt[e] - D;
+                        gx[e] += fmaf(diff, mu[m][e], D);
+                        acc[m][e] = fmaf(xs[e], diff, acc[m][e]);
                     }
                 }
                 if constexpr (sizeof(IO) * VEC == 16) store_vec_nt<IO, VEC>(gx_ + slab + (size_t)tt[j] * C, gx);
@@ -220,9 +223,14 @@ template <typename IO, int VEC>
 int launch_bwd(const void* x, const float* mix, const void* const* gout, void* gx, float* gmix, float* part, int n_mix,
                int B, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid, hipStream_t st) {
     const int ncv = C / VEC;
-    const int n_tchunk = (T + QS_TCH - 1) / QS_TCH;
     const dim3 block(QS_CX * QS_TY);
     const int gbx = (ncv + QS_CX - 1) / QS_CX;
+    // Token chunks: as many as give about QS_TARGET_WG workgroups (one round of long-lived workgroups: measured at
+    // 64 x 196 x 768 bf16, three mixes, 40 us with 32-token chunks, 30 us with two chunks of 98), at most one per 32
+    // tokens (the workspace's row count), at least one.
+    const int max_tchunk = (T + QS_TCH - 1) / QS_TCH;
+    int n_tchunk = (int)((QS_TARGET_WG + (long long)gbx * B / 2) / ((long long)gbx * B));
+    n_tchunk = n_tchunk < 1 ? 1 : n_tchunk > max_tchunk ? max_tchunk : n_tchunk;
     if ((long long)gbx * n_tchunk * B > 0x7fffffffLL) {
         set_error("qshift_mix_bwd: too many workgroups (%d x %d x %d)", gbx, n_tchunk, B);
         return VRWKV_UNSUPPORTED_SHAPE;
@@ -248,7 +256,9 @@ int launch_bwd(const void* x, const float* mix, const void* const* gout, void* g
 template <typename IO>
 int launch_bwd_io(const void* x, const float* mix, const void* const* gout, void* gx, float* gmix, float* part, int n_mix,
                   int B, int T, int C, int Hp, int Wp, int shift, int g, int head_dim, int n_grid, bool vec_ok, hipStream_t st) {
-    constexpr int V = 16 / sizeof(IO);
+    // four channels per thread: 16-byte accesses of fp32, 8-byte ones of 16-bit elements (eight channels per thread
+    // cost 153 registers with three mixes, three waves per SIMD: measured 10-13 % slower)
+    constexpr int V = 4;
     const int period = head_dim > 0 ? head_dim : C;
     if (vec_ok && C % V == 0 && g % V == 0 && period % V == 0)
         return launch_bwd<IO, V>(x, mix, gout, gx, gmix, part, n_mix, B, T, C, Hp, Wp, shift, g, head_dim, n_grid, st);
