@@ -49,8 +49,10 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 // W waves share a row (1: a wave per row, short rows; 4: the workgroup's four waves, long rows), a thread keeps VPL
 // 16-byte vectors of it.  A group takes R rows whose loads are all issued before the first value is used, so a thread
-// has 2 x 16 bytes x VPL x R in flight; workgroups are short and many, the dispatcher evens out the load.
-template <int VPL> constexpr int rows_per_group_fwd() { return VPL <= 2 ? 2 : 1; }
+// has 2 x 16 bytes x VPL x R in flight; workgroups are short and many, the dispatcher evens out the load.  R = 2 for
+// short rows, but 1 where a wave has a 16-bit row to itself (768 channels, sigmoid gate: 13.4 us with two rows per wave,
+// 12.1 us with one; four rows 15.6 us; a resident grid of 1024 workgroups walking the rows: no difference).
+template <int VPL, int ES, int W> constexpr int rows_per_group_fwd() { return VPL <= 2 && (ES == 4 || W > 1) ? 2 : 1; }
 
 template <typename IO, int VPL, int W, int PRE, int POST, bool HAS_LN>
 __global__ __launch_bounds__(256)
@@ -59,7 +61,7 @@ void rowfuse_kernel(const IO* __restrict__ a_, const IO* __restrict__ other_, co
                     long long rows, int N, float eps)
 {
     constexpr int V = 16 / (int)sizeof(IO);
-    constexpr int R = rows_per_group_fwd<VPL>();
+    constexpr int R = rows_per_group_fwd<VPL, (int)sizeof(IO), W>();
     constexpr int GROUP = WAVE * W;                            // threads per row
     __shared__ float s_red[W > 1 ? 2 * R : 1][4];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
@@ -519,7 +521,7 @@ int launch_bwd_io(const void* a, const void* other, const void* lnw, const void*
 template <typename IO, int VPL, int W, int PRE, int POST>
 int launch_ln(const void* a, const void* other, const void* lnw, const void* lnb, const void* gamma, void* out,
               long long rows, int N, float eps, hipStream_t st) {
-    constexpr int per_wg = (W == 1 ? 4 : 1) * rows_per_group_fwd<VPL>();
+    constexpr int per_wg = (W == 1 ? 4 : 1) * rows_per_group_fwd<VPL, (int)sizeof(IO), W>();
     if ((rows + per_wg - 1) / per_wg > 0x7fffffffLL) {
         set_error("rowfuse: too many rows (%lld)", rows);
         return VRWKV_UNSUPPORTED_SHAPE;
