@@ -511,9 +511,18 @@ def maa_mix(x, sx, m, maas, maa_table=None):
 
 
 def groupnorm_gate_tensor_ops(y, gate, gn_weight, gn_bias, n_groups, eps=1e-5):
-    """vrwkv6.py:205-211 and :199: ln_x on the (B*T, C) view, times silu(gate)."""
+    """vrwkv6.py:205-211 and :199: ln_x on the (B*T, C) view, times silu(gate).  The group statistics are written out
+    with mean / var instead of torch.nn.functional.group_norm: on a GPU that function's backward returns wrong weight
+    and bias gradients for a 2-D input of more than 128 rows (PyTorch 2.10.0+rocm7.0, every dtype: measured against
+    the sums written out in float64 and against the CPU), and this function is the path that autograd differentiates
+    when the kernels do not apply.  Statistics in fp32 for 16-bit inputs, as the library computes them."""
     C = y.shape[-1]
-    yn = torch.nn.functional.group_norm(y.to(gate.dtype).reshape(-1, C), n_groups, gn_weight, gn_bias, eps)
+    x = y.to(gate.dtype).reshape(-1, n_groups, C // n_groups)
+    xs = x.float() if x.dtype in (torch.bfloat16, torch.float16) else x
+    mean = xs.mean(-1, keepdim=True)
+    var = xs.var(-1, unbiased=False, keepdim=True)
+    xh = ((xs - mean) * torch.rsqrt(var + eps)).reshape(-1, C)
+    yn = (xh * gn_weight + gn_bias).to(gate.dtype)
     return yn.view(gate.shape) * torch.nn.functional.silu(gate)
 
 
