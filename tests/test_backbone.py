@@ -156,6 +156,57 @@ def test_vrwkv6_backbone_fused_equals_eager_and_trains(cls):
     assert net.layers[0].att.time_faaaa.grad.abs().sum().item() > 0
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["vrwkv", "vrwkv_key_norm", "vrwkv6", "vrwkv6_cls"])
+def test_every_parameter_gradient_fused_equals_tensor_ops(kind):
+    """One training step of a two-block backbone on 3 x 140 (141) tokens in fp32: the gradient of every parameter
+    with the element-wise steps on the HIP kernels and their hand-written backward kernels against the same model
+    with those steps as PyTorch tensor ops under autograd (the WKV operators are the HIP ones in both).  More than
+    128 rows, so the channel sums of every backward kernel span several partial rows.
+    Tolerance: 2e-4 of each gradient's largest entry (fast exp / rcp in the gates, fp32 sums in another order)."""
+    import vision_rwkv_amd as ops
+    torch.manual_seed(4)
+    if kind.startswith("vrwkv6"):
+        cls = kind.endswith("cls")
+        net = ops.VRWKV6(img_size=64, embed_dims=128, num_heads=2, depth=2, post_norm=True, init_values=0.1,
+                         with_cls_token=cls, output_cls_token=cls).cuda()
+    else:
+        cls = False
+        net = ops.VRWKV(img_size=64, embed_dims=128, depth=2, post_norm=not kind.endswith("key_norm"), init_values=0.1,
+                        key_norm=kind.endswith("key_norm")).cuda()
+    for prm in net.parameters():                      # layer scales and biases away from their initial values
+        if prm.dim() == 1:
+            prm.data.add_(0.1 * torch.randn_like(prm))
+    img = torch.randn(3, 3, 224, 160).cuda()
+    net.train()
+
+    def grads():
+        net.zero_grad(set_to_none=True)
+        out = net(img)
+        out = out[0] if cls else out
+        (out * torch.linspace(-1, 1, out.numel(), device=out.device).view_as(out)).sum().backward()
+        return {n: p.grad.clone() for n, p in net.named_parameters() if p.grad is not None}, out.detach()
+
+    g_fused, y_fused = grads()
+    for m in net.modules():
+        if hasattr(m, "fused_shift"):
+            m.fused_shift = False
+    ops.ops.ROW_FUSE_ENABLED = False
+    try:
+        g_eager, y_eager = grads()
+    finally:
+        ops.ops.ROW_FUSE_ENABLED = True
+    assert (y_fused - y_eager).abs().max().item() <= 1e-4 * y_eager.abs().max().item()
+    assert set(g_fused) == set(g_eager) and len(g_fused) > 20
+    worst = ("", 0.0)
+    for name, ge in g_eager.items():
+        err = (g_fused[name] - ge).abs().max().item() / max(ge.abs().max().item(), 1e-12)
+        if err > worst[1]:
+            worst = (name, err)
+        assert err <= 2e-4, (name, err)
+    print(f"  {kind}: {len(g_eager)} parameter gradients, worst {worst[0]} {worst[1]:.1e}")
+
+
 @pytest.mark.parametrize("kind", ["vrwkv", "vrwkv6"])
 def test_reference_checkpoint_keys_load(kind):
     """CPU: a state dict with the reference's key names (vrwkv.py:351-358 keeps the patch embedding as
