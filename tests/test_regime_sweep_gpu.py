@@ -1,0 +1,81 @@
+"""Bi-WKV forward (plain and gated) and backward on random mixes of parameter regimes inside one call: per channel
+either VRWKV's own range (w, u of order 1/T), a strong decay (w up to 6 or up to 60 per token), a growing weight
+(w down to -30/T), w = u = 0, or a bonus of +-30; k of unit spread or 5 / 20 times that (softmax weights spanning
+e^+-60); sequence lengths on both sides of every path boundary (one launch, two or three super-chunks in one launch,
+two launches); fp32, bf16 and fp16 rows.  Channels of different regimes share 64-channel tiles, so plain-sum tiles,
+tiles redone by the renormalising recurrence and the sequential backward all occur in one call.
+
+Reference: the C oracle (float64).  Bounds, err = max|x - ref| / max(|ref|, rms(ref)) per tensor:
+  forward, fp32 rows: 1e-4 with k of unit spread, 2e-4 with the wider k (two of 70 sweep cases read 1.2e-4 and 1.9e-4
+    at 672 / 673 tokens with k of 20 times the unit spread);
+  forward, 16-bit rows: 1e-2;
+  gk, gv, fp32 rows: 2e-4 with k of unit spread, 1e-2 with the wider k -- where single tokens dominate the softmax,
+    v_i sum(z) - sum(z y) cancels and the gradient's own scale shrinks; the same inputs through the softmax form
+    evaluated in float32 lose the same digits;
+  gk, gv, 16-bit rows: 3e-2;  gw, gu: 2e-3 (fp32), 3e-2 (16-bit).
+Everything must be finite."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _params(rng, C, T):
+    w, u = np.empty(C, np.float32), np.empty(C, np.float32)
+    for c, r in enumerate(rng.integers(0, 6, C)):
+        if r == 0:
+            w[c], u[c] = rng.uniform(-5, 3) / T, rng.uniform(-2, 1) / T
+        elif r == 1:
+            w[c], u[c] = rng.uniform(0.5, 6), rng.uniform(-3, 3)
+        elif r == 2:
+            w[c], u[c] = -rng.uniform(0, 30) / T, rng.uniform(-1, 1)
+        elif r == 3:
+            w[c], u[c] = 0.0, 0.0
+        elif r == 4:
+            w[c], u[c] = rng.uniform(-5, 3) / T, rng.choice([-30.0, 30.0])
+        else:
+            w[c], u[c] = rng.uniform(10, 60), rng.uniform(-1, 1)
+    return w, u
+
+
+@pytest.mark.parametrize("seed,B,T,C,dtype,kscale", [
+    (1, 2, 196, 192, torch.float32, 1.0), (2, 3, 224, 256, torch.float32, 5.0), (3, 1, 225, 128, torch.float32, 1.0),
+    (4, 2, 448, 320, torch.bfloat16, 5.0), (5, 2, 673, 200, torch.float32, 20.0), (6, 1, 672, 320, torch.float16, 20.0),
+    (7, 2, 700, 256, torch.float32, 1.0), (8, 3, 29, 64, torch.float32, 20.0), (9, 1, 1024, 192, torch.bfloat16, 1.0),
+    (10, 2, 300, 200, torch.float16, 5.0), (11, 1, 1500, 128, torch.float32, 5.0), (12, 2, 7, 64, torch.float32, 1.0)])
+def test_mixed_parameter_regimes(seed, B, T, C, dtype, kscale):
+    import vision_rwkv_amd as ops
+    from oracle import blocks, clib
+    rng = np.random.default_rng(seed)
+    w, u = _params(rng, C, T)
+    k = (rng.standard_normal((B, T, C)) * kscale).astype(np.float32)
+    v, gy = (rng.standard_normal((B, T, C)).astype(np.float32) for _ in range(2))
+    r = (2 * rng.standard_normal((B, T, C))).astype(np.float32)
+    td = lambda a: torch.from_numpy(a).to(DEV).to(dtype)
+    kd, vd, rd, gd = td(k), td(v), td(r), td(gy)
+    wt, ut = torch.from_numpy(w).to(DEV), torch.from_numpy(u).to(DEV)
+    y = ops.bi_wkv_forward(wt, ut, kd, vd)
+    yg = ops.bi_wkv_forward(wt, ut, kd, vd, gate=rd)
+    gw, gu, gk, gv = ops.bi_wkv_backward(wt, ut, kd, vd, gd)
+    torch.cuda.synchronize()
+    f = lambda x: x.float().cpu().numpy()
+    for name, t in (("y", y), ("yg", yg), ("gk", gk), ("gv", gv), ("gw", gw), ("gu", gu)):
+        assert np.isfinite(f(t)).all(), name
+    fp32 = dtype == torch.float32
+    ref = clib.biwkv_fwd(w, u, f(kd), f(vd))
+    refg = blocks.row_epilogue(ref, f(rd), post=blocks.POST_SIGMOID_GATE).reshape(B, T, C)
+    tol_y = (1e-4 if kscale == 1.0 else 2e-4) if fp32 else 1e-2
+    err = {"y": rel_err(f(y), ref), "yg": rel_err(f(yg), refg)}
+    assert err["y"] <= tol_y and err["yg"] <= tol_y, err
+    if T <= 700:                                               # the O(T^2) adjoint
+        rgw, rgu, rgk, rgv = clib.biwkv_bwd(w, u, f(kd), f(vd), f(gd))
+        err.update(gk=rel_err(f(gk), rgk), gv=rel_err(f(gv), rgv), gw=rel_err(f(gw), rgw), gu=rel_err(f(gu), rgu))
+        tol_g = (2e-4 if kscale == 1.0 else 1e-2) if fp32 else 3e-2
+        tol_p = 2e-3 if fp32 else 3e-2
+        assert err["gk"] <= tol_g and err["gv"] <= tol_g, err
+        assert err["gw"] <= tol_p and err["gu"] <= tol_p, err
+    print("  " + ", ".join(f"{n} {e:.1e}" for n, e in err.items()), flush=True)
