@@ -515,6 +515,33 @@ def backbone_section(torch, ops, steps, warmup):
         netb(imgb).float().square().mean().backward()
 
     ms_train = timed(train_step, max(steps // 2, 3), max(warmup // 4, 3))
+    # the same step recorded once as a HIP graph and replayed (every kernel of the build launches on the stream it is
+    # given and allocates nothing, so the whole forward + backward can be captured); the gradients of a replay are
+    # compared with the eager step's on the same images
+    graph_step = {"ms_per_step": None}
+    try:
+        params = [p for p in netb.parameters() if p.requires_grad]
+        train_step()
+        torch.cuda.synchronize()
+        eager_grads = [p.grad.clone() for p in params]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                train_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        netb.zero_grad(set_to_none=True)
+        with torch.cuda.graph(graph):
+            netb(imgb).float().square().mean().backward()
+        ms_graph = timed(graph.replay, max(steps // 2, 3), 3)
+        same = all(torch.equal(p.grad, g) for p, g in zip(params, eager_grads))
+        graph_step = {"ms_per_step": round(ms_graph, 3), "images_per_s": round(64 / ms_graph * 1e3, 1),
+                      "gradients_equal_the_eager_step": bool(same)}
+        del graph
+    except Exception as exc:                                   # reported, never fatal for the headline
+        graph_step["error"] = f"{type(exc).__name__}: {exc}"[:200]
     del netb
     net6t = ops.vrwkv6_b().to(dev).bfloat16()
     net6t.train()
@@ -536,7 +563,8 @@ def backbone_section(torch, ops, steps, warmup):
                         "ms_per_forward_gate_as_a_pass_of_its_own": round(ms_b_fwd_gate_pass, 3)},
             "vrwkv_b_train": {"workload": "VRWKV-B forward + backward (no optimizer step), batch 64, 224x224, T=196, C=768, "
                                           "12 blocks, bf16, random weights, Bi-WKV forward and backward on the HIP kernels",
-                              "ms_per_step": round(ms_train, 3), "images_per_s": round(64 / ms_train * 1e3, 1)},
+                              "ms_per_step": round(ms_train, 3), "images_per_s": round(64 / ms_train * 1e3, 1),
+                              "recorded_as_one_hip_graph_and_replayed": graph_step},
             "vrwkv6_b_train": {"workload": "VRWKV6-B forward + backward (no optimizer step), batch 64, 224x224, T=196, C=768, "
                                            "12 heads, 12 blocks, bf16, random weights, wkv6 forward and backward on the HIP kernels",
                                "ms_per_step": round(ms_train6, 3), "images_per_s": round(64 / ms_train6 * 1e3, 1)},
